@@ -1,0 +1,78 @@
+"""Builds the two shared libraries of the package, in-tree, for gfx950.
+
+``libkvmove.so``        hand-written HIP kernels + the C ABI (``include/kvmove.h``); no torch.
+``libkvmove_torch.so``  torch op shim registering ``block_migration_ops`` / ``swapping_ops``.
+
+Run as ``python -m distserve_amd.build``.  hipcc cross-compiles without a GPU.
+"""
+from __future__ import annotations
+
+import os
+import shutil
+import subprocess
+import sys
+
+PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+REPO_DIR = os.path.dirname(PKG_DIR)
+CSRC_DIR = os.path.join(PKG_DIR, "csrc")
+LIB_DIR = os.path.join(PKG_DIR, "lib")
+INCLUDE_DIR = os.path.join(REPO_DIR, "include")
+
+KVMOVE_LIB = os.path.join(LIB_DIR, "libkvmove.so")
+TORCH_LIB = os.path.join(LIB_DIR, "libkvmove_torch.so")
+
+GPU_ARCH = "gfx950"
+ROCM_HOME = os.environ.get("ROCM_PATH", "/opt/rocm")
+
+
+def _run(cmd):
+    print("+", " ".join(cmd), flush=True)
+    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    # the host pass of hipcc does not know the packed-fp32 target feature and says so
+    out = "\n".join(l for l in res.stdout.splitlines() if "packed-fp32-ops" not in l)
+    if out.strip():
+        print(out, flush=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"build step failed with exit code {res.returncode}: {' '.join(cmd)}")
+
+
+def build_kvmove() -> str:
+    hipcc = shutil.which("hipcc") or os.path.join(ROCM_HOME, "bin", "hipcc")
+    os.makedirs(LIB_DIR, exist_ok=True)
+    _run([
+        hipcc, f"--offload-arch={GPU_ARCH}", "-O3", "-std=c++17", "-fPIC", "-shared",
+        "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+        "-Wall", "-Wextra", f"-I{INCLUDE_DIR}",
+        os.path.join(CSRC_DIR, "kvmove.hip"), "-o", KVMOVE_LIB,
+    ])
+    return KVMOVE_LIB
+
+
+def build_torch_shim() -> str:
+    import torch
+    from torch.utils import cpp_extension
+
+    if not os.path.exists(KVMOVE_LIB):
+        build_kvmove()
+    torch_lib_dir = os.path.join(os.path.dirname(torch.__file__), "lib")
+    cmd = ["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall",
+           "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1",
+           f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}",
+           f"-I{INCLUDE_DIR}", f"-I{os.path.join(ROCM_HOME, 'include')}"]
+    cmd += [f"-I{p}" for p in cpp_extension.include_paths()]
+    cmd += [os.path.join(CSRC_DIR, "kvmove_torch.cpp"), "-o", TORCH_LIB,
+            f"-L{LIB_DIR}", "-lkvmove", "-Wl,-rpath,$ORIGIN",
+            f"-L{torch_lib_dir}", "-lc10", "-lc10_hip", "-ltorch_cpu", "-ltorch", "-Wl,--no-as-needed"]
+    _run(cmd)
+    return TORCH_LIB
+
+
+def build_all() -> None:
+    build_kvmove()
+    build_torch_shim()
+
+
+if __name__ == "__main__":
+    build_all()
+    print("built:", KVMOVE_LIB, TORCH_LIB)
+    sys.exit(0)

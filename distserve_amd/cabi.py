@@ -1,0 +1,162 @@
+"""ctypes binding of the kvmove C ABI (``include/kvmove.h``), one Python function per entry point.
+
+Pointers are plain integers (``tensor.data_ptr()``), streams are ``hipStream_t`` values as
+integers (``torch.cuda.current_stream().cuda_stream``).  A nonzero return code raises
+``KvmError`` carrying ``kvm_last_error()``.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from typing import List, Sequence
+
+KVM_OK = 0
+KVM_EINVAL = -1
+KVM_ERANGE = -2
+KVM_EDUP = -3
+KVM_ENOTREG = -4
+KVM_EHIP = -5
+KVM_EHANDLE = -6
+KVM_EMISMATCH = -7
+KVM_HANDLE_WORDS = 8
+
+# every symbol include/kvmove.h declares
+EXPORTS = (
+    "kvm_version", "kvm_last_error", "kvm_get_mem_handle", "kvm_register_mem_handle",
+    "kvm_register_source", "kvm_reset", "kvm_migrate", "kvm_swap", "kvm_copy_plain",
+    "kvm_set_option", "kvm_get_option", "kvm_migrate_plan",
+)
+
+
+class KvmError(RuntimeError):
+    def __init__(self, code: int, text: str):
+        super().__init__(f"{text} (kvmove error {code})")
+        self.code = code
+
+
+class KvmGeom(ctypes.Structure):
+    _fields_ = [
+        ("num_layers", ctypes.c_int64), ("num_kv_heads", ctypes.c_int64), ("block_size", ctypes.c_int64),
+        ("head_dim", ctypes.c_int64), ("dtype_bytes", ctypes.c_int64),
+        ("ctx_pp_size", ctypes.c_int32), ("ctx_tp_size", ctypes.c_int32),
+        ("dec_pp_size", ctypes.c_int32), ("dec_tp_size", ctypes.c_int32),
+        ("dec_pp_rank", ctypes.c_int32), ("dec_tp_rank", ctypes.c_int32),
+    ]
+
+
+def _lib_path() -> str:
+    lib_dir = os.environ.get("KVMOVE_LIB_DIR") or os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib")
+    return os.path.join(lib_dir, "libkvmove.so")
+
+
+def _load() -> ctypes.CDLL:
+    path = _lib_path()
+    if not os.path.exists(path):
+        raise RuntimeError(f"libkvmove.so not found at {path}; build it with `python -m distserve_amd.build`")
+    lib = ctypes.CDLL(path)
+    i64, i32, vp, ip = ctypes.c_int64, ctypes.c_int32, ctypes.c_void_p, ctypes.POINTER(ctypes.c_int64)
+    lib.kvm_version.restype = ctypes.c_int
+    lib.kvm_last_error.restype = ctypes.c_char_p
+    lib.kvm_get_mem_handle.argtypes = [vp, i64, ip]
+    lib.kvm_register_mem_handle.argtypes = [ip, ip, i64, i64, ip, ip]
+    lib.kvm_register_source.argtypes = [i32, i32, i32, i32, i64, i64, vp, vp, i64]
+    lib.kvm_reset.argtypes = []
+    lib.kvm_migrate.argtypes = [ctypes.POINTER(KvmGeom), ip, ip, i64, vp, vp, i64, vp]
+    lib.kvm_swap.argtypes = [ip, ip, i64, ctypes.c_int, vp, vp, vp, vp, i64, i64, i64, vp]
+    lib.kvm_copy_plain.argtypes = [vp, vp, i64, vp]
+    lib.kvm_set_option.argtypes = [ctypes.c_char_p, i64]
+    lib.kvm_get_option.argtypes = [ctypes.c_char_p]
+    lib.kvm_get_option.restype = i64
+    lib.kvm_migrate_plan.argtypes = [ctypes.POINTER(KvmGeom), i64, vp, vp, ip]
+    for name in EXPORTS:
+        fn = getattr(lib, name)
+        if name not in ("kvm_last_error", "kvm_get_option", "kvm_version"):
+            fn.restype = ctypes.c_int
+    return lib
+
+
+lib = _load()
+
+
+def _check(rc: int) -> None:
+    if rc != KVM_OK:
+        raise KvmError(rc, lib.kvm_last_error().decode())
+
+
+def _arr(values: Sequence[int]):
+    return (ctypes.c_int64 * len(values))(*values)
+
+
+def version() -> int:
+    return lib.kvm_version()
+
+
+def geom(num_layers, num_kv_heads, block_size, head_dim, dtype_bytes, ctx_pp=1, ctx_tp=1,
+         dec_pp=1, dec_tp=1, dec_pp_rank=0, dec_tp_rank=0) -> KvmGeom:
+    return KvmGeom(num_layers, num_kv_heads, block_size, head_dim, dtype_bytes,
+                   ctx_pp, ctx_tp, dec_pp, dec_tp, dec_pp_rank, dec_tp_rank)
+
+
+def get_mem_handle(dev_ptr: int, nbytes: int) -> List[int]:
+    out = (ctypes.c_int64 * KVM_HANDLE_WORDS)()
+    _check(lib.kvm_get_mem_handle(dev_ptr, nbytes, out))
+    return list(out)
+
+
+def register_mem_handle(k_handle, v_handle, num_layers, num_kv_heads, context_pc, decoding_pc) -> None:
+    if len(k_handle) != KVM_HANDLE_WORDS or len(v_handle) != KVM_HANDLE_WORDS:
+        raise KvmError(KVM_EHANDLE, f"a memory handle has {KVM_HANDLE_WORDS} words")
+    if len(context_pc) != 4 or len(decoding_pc) != 4:
+        raise KvmError(KVM_EINVAL, "parallel configs are [tp_size, tp_rank, pp_size, pp_rank]")
+    _check(lib.kvm_register_mem_handle(_arr(k_handle), _arr(v_handle), num_layers, num_kv_heads,
+                                       _arr(context_pc), _arr(decoding_pc)))
+
+
+def register_source(ctx_pp_size, ctx_tp_size, pp_rank, tp_rank, num_layers, num_kv_heads,
+                    k_ptr: int, v_ptr: int, nbytes_each: int) -> None:
+    _check(lib.kvm_register_source(ctx_pp_size, ctx_tp_size, pp_rank, tp_rank, num_layers, num_kv_heads,
+                                   k_ptr, v_ptr, nbytes_each))
+
+
+def reset() -> None:
+    _check(lib.kvm_reset())
+
+
+def migrate(g: KvmGeom, ctx_idx: Sequence[int], dec_idx: Sequence[int], dst_k: int, dst_v: int,
+            dst_num_blocks: int, stream: int = 0, n: int | None = None) -> None:
+    n = len(ctx_idx) if n is None else n
+    if n == len(ctx_idx) and len(ctx_idx) != len(dec_idx):
+        raise KvmError(KVM_EINVAL, f"{len(ctx_idx)} context blocks but {len(dec_idx)} decoding blocks")
+    _check(lib.kvm_migrate(ctypes.byref(g), _arr(ctx_idx), _arr(dec_idx), n, dst_k, dst_v,
+                           dst_num_blocks, stream))
+
+
+def swap(src_ids: Sequence[int], dst_ids: Sequence[int], is_swap_in: bool, k_gpu: int, v_gpu: int,
+         k_host: int, v_host: int, slab_bytes: int, n_gpu_blocks: int, n_host_blocks: int,
+         stream: int = 0) -> None:
+    if len(src_ids) != len(dst_ids):
+        raise KvmError(KVM_EINVAL, f"{len(src_ids)} source blocks but {len(dst_ids)} target blocks")
+    _check(lib.kvm_swap(_arr(src_ids), _arr(dst_ids), len(src_ids), 1 if is_swap_in else 0, k_gpu, v_gpu,
+                        k_host, v_host, slab_bytes, n_gpu_blocks, n_host_blocks, stream))
+
+
+def copy_plain(dst: int, src: int, nbytes: int, stream: int = 0) -> None:
+    _check(lib.kvm_copy_plain(dst, src, nbytes, stream))
+
+
+def set_option(name: str, value: int) -> None:
+    _check(lib.kvm_set_option(name.encode(), value))
+
+
+def get_option(name: str) -> int:
+    v = lib.kvm_get_option(name.encode())
+    if v == KVM_EINVAL and lib.kvm_last_error():
+        raise KvmError(KVM_EINVAL, lib.kvm_last_error().decode())
+    return v
+
+
+def migrate_plan(g: KvmGeom, n: int, dst_k: int, dst_v: int) -> dict:
+    out = (ctypes.c_int64 * 6)()
+    _check(lib.kvm_migrate_plan(ctypes.byref(g), n, dst_k, dst_v, out))
+    keys = ("workgroups_per_block", "threads", "vector_bytes", "segments", "launches", "payload_bytes_per_block")
+    return dict(zip(keys, list(out)))

@@ -1,0 +1,808 @@
+// kvmove.hip -- KV-block migration and swap for MI355X (gfx950, wave64).
+//
+// The whole path is byte movement, so there is no MFMA here.  One copy kernel serves
+// migration (gather by block-index tables + re-slice of layers/heads between the context
+// instance's TP/PP layout and one decoding rank), the kernel flavour of swap, and the
+// plain calibration copy.  Its metadata (segment table and block-index pairs) travels in
+// the kernel-argument segment, so every workgroup picks it up with scalar loads into
+// SGPRs and no device-side table, staging copy or allocation exists anywhere on the path.
+//
+// Reference call sites this stands behind: distserve/worker.py:133-134 (handles),
+// :239-246 (registration), :250-267 (migrate_blocks), :303-311 (swap).
+#include "kvmove.h"
+
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <atomic>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <string>
+#include <tuple>
+#include <vector>
+#include <unistd.h>
+
+namespace {
+
+// ------------------------------------------------------------------ kernel argument
+
+constexpr int kMaxSegs = 8;    // source segments per launch
+constexpr int kMaxIdx = 440;   // block-index pairs per launch (keeps the argument <= 4 KiB)
+
+// One rectangle of the decoding rank's block that a single context rank supplies:
+// n_rows runs of run_bytes, one per overlapping layer.
+struct Seg {
+    const char *src_k;         // context pool base + offset of the rectangle inside a block
+    const char *src_v;
+    uint64_t src_block_stride; // bytes per source block
+    uint32_t src_row_stride;   // bytes between consecutive layers in the source block
+    uint32_t dst_row_stride;   // ... in the destination block
+    uint32_t dst_off;          // offset of the rectangle inside a destination block
+    uint32_t run_bytes;        // contiguous bytes per row
+    uint32_t n_rows;
+    uint32_t rows_per_tile;    // >1 only when a whole row is smaller than a tile
+    uint32_t pieces_per_row;   // >1 only when a row is larger than a tile
+    uint32_t piece_bytes;
+    uint32_t tile_end;         // exclusive prefix sum of tiles over the launch's segments
+    uint32_t pad_;
+};
+static_assert(sizeof(Seg) == 64, "Seg layout");
+
+struct IdxPair {
+    int32_t ctx;  // block in the context pools
+    int32_t dec;  // block in the decoding pool
+};
+
+struct MigrateArgs {
+    char *dst_k;
+    char *dst_v;
+    uint64_t dst_block_stride;
+    uint32_t nseg;
+    uint32_t nidx;
+    Seg seg[kMaxSegs];
+    IdxPair idx[kMaxIdx];
+};
+static_assert(sizeof(MigrateArgs) <= 4096, "kernel argument must stay within 4 KiB");
+
+// ------------------------------------------------------------------------- device
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+template <bool NT, typename V>
+__device__ __forceinline__ V ld(const V *p)
+{
+    if constexpr (NT) return __builtin_nontemporal_load(p);
+    else return *p;
+}
+
+template <bool NT, typename V>
+__device__ __forceinline__ void st(V *p, V v)
+{
+    if constexpr (NT) __builtin_nontemporal_store(v, p);
+    else *p = v;
+}
+
+// One contiguous run of `len` bytes (a multiple of sizeof(V)) by the whole workgroup:
+// UNROLL independent 16-byte loads per lane are issued before the first store.
+template <typename V, int THREADS, int UNROLL, bool NTL, bool NTS>
+__device__ __forceinline__ void copy_run(char *dst, const char *src, uint32_t len)
+{
+    constexpr uint32_t kPass = THREADS * (uint32_t)sizeof(V);
+    constexpr uint32_t kStep = kPass * UNROLL;
+    const uint32_t lane_off = threadIdx.x * (uint32_t)sizeof(V);
+    uint32_t off = 0;
+    for (; off + kStep <= len; off += kStep) {
+        V r[UNROLL];
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u)
+            r[u] = ld<NTL>(reinterpret_cast<const V *>(src + off + u * kPass + lane_off));
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u)
+            st<NTS>(reinterpret_cast<V *>(dst + off + u * kPass + lane_off), r[u]);
+    }
+    if (off < len) {
+        V r[UNROLL];
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            const uint32_t o = off + u * kPass + lane_off;
+            if (o < len) r[u] = ld<NTL>(reinterpret_cast<const V *>(src + o));
+        }
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            const uint32_t o = off + u * kPass + lane_off;
+            if (o < len) st<NTS>(reinterpret_cast<V *>(dst + o), r[u]);
+        }
+    }
+}
+
+// `nrows` runs of `len` bytes each, `sstride` / `dstride` apart: the UNROLL loads in
+// flight span row boundaries, so short rows still keep several loads outstanding.
+// The (row, pass-in-row) counters are wave-uniform and advance in SGPRs.
+template <typename V, int THREADS, int UNROLL, bool NTL, bool NTS>
+__device__ __forceinline__ void copy_rows(char *dst, const char *src, uint32_t nrows, uint32_t len,
+                                          uint32_t sstride, uint32_t dstride)
+{
+    constexpr uint32_t kPass = THREADS * (uint32_t)sizeof(V);
+    const uint32_t lane_off = threadIdx.x * (uint32_t)sizeof(V);
+    const uint32_t passes_per_row = (len + kPass - 1) / kPass;
+    const uint32_t total_passes = nrows * passes_per_row;
+    uint32_t row = 0, pc = 0;
+    for (uint32_t q = 0; q < total_passes; q += UNROLL) {
+        V r[UNROLL];
+        uint32_t soff[UNROLL], doff[UNROLL];
+        bool ok[UNROLL];
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            const uint32_t col = pc * kPass + lane_off;
+            ok[u] = (row < nrows) && (col < len);
+            soff[u] = row * sstride + col;
+            doff[u] = row * dstride + col;
+            if (++pc == passes_per_row) { pc = 0; ++row; }
+        }
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u)
+            if (ok[u]) r[u] = ld<NTL>(reinterpret_cast<const V *>(src + soff[u]));
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u)
+            if (ok[u]) st<NTS>(reinterpret_cast<V *>(dst + doff[u]), r[u]);
+    }
+}
+
+// grid = (tiles per block of one pool kind, blocks in this launch, 2 = {K, V}).
+// Everything up to the lane offset is wave-uniform: the segment, the block-index pair and
+// the tile's base addresses are scalar loads from the kernel-argument segment into SGPRs.
+template <typename V, int THREADS, int UNROLL, bool NTL, bool NTS>
+__global__ __launch_bounds__(THREADS) void kvm_copy_kernel(const MigrateArgs a)
+{
+    uint32_t tile = blockIdx.x;
+    uint32_t s = 0, tile_begin = 0;
+    while (s + 1 < a.nseg && tile >= a.seg[s].tile_end) {
+        tile_begin = a.seg[s].tile_end;
+        ++s;
+    }
+    tile -= tile_begin;
+    const Seg &sg = a.seg[s];
+    const IdxPair ix = a.idx[blockIdx.y];
+    const bool is_v = blockIdx.z != 0;
+
+    const char *src = (is_v ? sg.src_v : sg.src_k) + (uint64_t)(uint32_t)ix.ctx * sg.src_block_stride;
+    char *dst = (is_v ? a.dst_v : a.dst_k) + (uint64_t)(uint32_t)ix.dec * a.dst_block_stride + sg.dst_off;
+
+    if (sg.rows_per_tile == 1) {
+        const uint32_t row = tile / sg.pieces_per_row;
+        const uint32_t piece = tile - row * sg.pieces_per_row;
+        const uint32_t col_off = piece * sg.piece_bytes;
+        const uint32_t len = min(sg.piece_bytes, sg.run_bytes - col_off);
+        copy_run<V, THREADS, UNROLL, NTL, NTS>(dst + (uint64_t)row * sg.dst_row_stride + col_off,
+                                               src + (uint64_t)row * sg.src_row_stride + col_off, len);
+    } else {
+        const uint32_t row0 = tile * sg.rows_per_tile;
+        const uint32_t nrows = min(sg.rows_per_tile, sg.n_rows - row0);
+        copy_rows<V, THREADS, UNROLL, NTL, NTS>(dst + (uint64_t)row0 * sg.dst_row_stride,
+                                                src + (uint64_t)row0 * sg.src_row_stride, nrows,
+                                                sg.run_bytes, sg.src_row_stride, sg.dst_row_stride);
+    }
+}
+
+// --------------------------------------------------------------------------- host
+
+thread_local std::string g_err;
+
+int fail(int code, const char *fmt, ...)
+{
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof buf, fmt, ap);
+    va_end(ap);
+    g_err = buf;
+    return code;
+}
+
+#define KVM_HIP(expr)                                                                          \
+    do {                                                                                       \
+        hipError_t e_ = (expr);                                                                \
+        if (e_ != hipSuccess)                                                                  \
+            return fail(KVM_EHIP, "%s failed: %s", #expr, hipGetErrorString(e_));              \
+    } while (0)
+
+// ---- options
+
+std::atomic<int64_t> opt_tile_bytes{32768};
+std::atomic<int64_t> opt_threads{256};
+std::atomic<int64_t> opt_unroll{4};
+std::atomic<int64_t> opt_nt_load{1};
+std::atomic<int64_t> opt_nt_store{1};
+std::atomic<int64_t> opt_swap_mode{0};
+
+std::atomic<int64_t> *find_opt(const char *name)
+{
+    if (!name) return nullptr;
+    if (!strcmp(name, "tile_bytes")) return &opt_tile_bytes;
+    if (!strcmp(name, "threads")) return &opt_threads;
+    if (!strcmp(name, "unroll")) return &opt_unroll;
+    if (!strcmp(name, "nt_load")) return &opt_nt_load;
+    if (!strcmp(name, "nt_store")) return &opt_nt_store;
+    if (!strcmp(name, "swap_mode")) return &opt_swap_mode;
+    return nullptr;
+}
+
+// ---- registry of context pools, keyed by (pp_rank, tp_rank)
+
+struct Source {
+    int32_t ctx_pp_size, ctx_tp_size;
+    int64_t num_layers, num_kv_heads;
+    const char *k, *v;
+    int64_t nbytes;
+};
+
+std::mutex g_mu;
+std::map<std::pair<int32_t, int32_t>, Source> g_sources;
+
+constexpr int64_t kHandleMagic = 0x4b564d4f56453031LL;  // "KVMOVE01"
+
+// ---- kernel table
+
+using KernelFn = void (*)(const MigrateArgs);
+
+template <typename V>
+KernelFn pick_narrow()
+{
+    return kvm_copy_kernel<V, 256, 4, true, true>;
+}
+
+template <int THREADS, int UNROLL>
+KernelFn pick_nt(bool ntl, bool nts)
+{
+    if (ntl) return nts ? kvm_copy_kernel<u32x4, THREADS, UNROLL, true, true>
+                        : kvm_copy_kernel<u32x4, THREADS, UNROLL, true, false>;
+    return nts ? kvm_copy_kernel<u32x4, THREADS, UNROLL, false, true>
+               : kvm_copy_kernel<u32x4, THREADS, UNROLL, false, false>;
+}
+
+template <int THREADS>
+KernelFn pick_unroll(int unroll, bool ntl, bool nts)
+{
+    switch (unroll) {
+    case 1: return pick_nt<THREADS, 1>(ntl, nts);
+    case 2: return pick_nt<THREADS, 2>(ntl, nts);
+    case 8: return pick_nt<THREADS, 8>(ntl, nts);
+    default: return pick_nt<THREADS, 4>(ntl, nts);
+    }
+}
+
+struct Launch {
+    KernelFn fn;
+    int threads;
+    int vec;
+};
+
+Launch pick_kernel(int vec)
+{
+    Launch l;
+    l.vec = vec;
+    if (vec != 16) {
+        l.threads = 256;
+        l.fn = vec == 8 ? pick_narrow<u32x2>()
+             : vec == 4 ? pick_narrow<uint32_t>()
+             : vec == 2 ? pick_narrow<uint16_t>()
+                        : pick_narrow<uint8_t>();
+        return l;
+    }
+    const int unroll = (int)opt_unroll.load();
+    const bool ntl = opt_nt_load.load() != 0, nts = opt_nt_store.load() != 0;
+    switch ((int)opt_threads.load()) {
+    case 512: l.threads = 512; l.fn = pick_unroll<512>(unroll, ntl, nts); break;
+    case 1024: l.threads = 1024; l.fn = pick_unroll<1024>(unroll, ntl, nts); break;
+    default: l.threads = 256; l.fn = pick_unroll<256>(unroll, ntl, nts); break;
+    }
+    return l;
+}
+
+int vec_width(uint64_t bits)
+{
+    // largest power of two <= 16 dividing every address and stride OR-ed into `bits`
+    for (int v = 16; v > 1; v >>= 1)
+        if ((bits & (uint64_t)(v - 1)) == 0) return v;
+    return 1;
+}
+
+// Splits a segment's rows into workgroup tiles of about tile_bytes.
+void tile_segment(Seg &s, uint32_t tile_bytes, uint32_t *tiles)
+{
+    if (s.run_bytes >= tile_bytes) {
+        s.rows_per_tile = 1;
+        s.piece_bytes = tile_bytes;
+        s.pieces_per_row = (s.run_bytes + tile_bytes - 1) / tile_bytes;
+        *tiles = s.n_rows * s.pieces_per_row;
+    } else {
+        s.rows_per_tile = std::max<uint32_t>(1, tile_bytes / s.run_bytes);
+        s.rows_per_tile = std::min(s.rows_per_tile, s.n_rows);
+        s.piece_bytes = s.run_bytes;
+        s.pieces_per_row = 1;
+        *tiles = (s.n_rows + s.rows_per_tile - 1) / s.rows_per_tile;
+    }
+}
+
+// Folds rows that are back to back on both sides into one long run.
+void collapse(Seg &s)
+{
+    if (s.n_rows > 1 && s.run_bytes == s.src_row_stride && s.run_bytes == s.dst_row_stride &&
+        (uint64_t)s.run_bytes * s.n_rows < (1ull << 32)) {
+        s.run_bytes *= s.n_rows;
+        s.src_row_stride = s.dst_row_stride = s.run_bytes;
+        s.n_rows = 1;
+    }
+}
+
+struct Plan {
+    std::vector<Seg> segs;         // untiled
+    int64_t min_src_blocks = 0;    // smallest block count over the pools that are read
+    uint64_t dst_block_stride = 0;
+    int vec = 16;
+    int64_t payload_per_block = 0; // K+V bytes this rank receives per block
+};
+
+int check_geom(const KvmGeom *g)
+{
+    if (!g) return fail(KVM_EINVAL, "geometry is null");
+    if (g->num_layers <= 0 || g->num_kv_heads <= 0 || g->block_size <= 0 || g->head_dim <= 0 ||
+        g->dtype_bytes <= 0)
+        return fail(KVM_EINVAL, "geometry has a non-positive dimension");
+    if (g->ctx_pp_size <= 0 || g->ctx_tp_size <= 0 || g->dec_pp_size <= 0 || g->dec_tp_size <= 0)
+        return fail(KVM_EINVAL, "parallel sizes must be positive");
+    if (g->dec_pp_rank < 0 || g->dec_pp_rank >= g->dec_pp_size || g->dec_tp_rank < 0 ||
+        g->dec_tp_rank >= g->dec_tp_size)
+        return fail(KVM_EINVAL, "decoding rank (pp %d, tp %d) outside (pp %d, tp %d)", g->dec_pp_rank,
+                    g->dec_tp_rank, g->dec_pp_size, g->dec_tp_size);
+    // distserve/config.py:281-285 and :252-256 assert the same divisibility
+    if (g->num_layers % g->ctx_pp_size || g->num_layers % g->dec_pp_size)
+        return fail(KVM_EINVAL, "num_layers %lld not divisible by a pipeline size (%d, %d)",
+                    (long long)g->num_layers, g->ctx_pp_size, g->dec_pp_size);
+    if (g->num_kv_heads % g->ctx_tp_size || g->num_kv_heads % g->dec_tp_size)
+        return fail(KVM_EINVAL, "num_kv_heads %lld not divisible by a tensor size (%d, %d)",
+                    (long long)g->num_kv_heads, g->ctx_tp_size, g->dec_tp_size);
+    return KVM_OK;
+}
+
+int build_plan(const KvmGeom *g, const void *dst_k, const void *dst_v, Plan *plan)
+{
+    if (int rc = check_geom(g)) return rc;
+    const int64_t Lc = g->num_layers / g->ctx_pp_size, Hc = g->num_kv_heads / g->ctx_tp_size;
+    const int64_t Ld = g->num_layers / g->dec_pp_size, Hd = g->num_kv_heads / g->dec_tp_size;
+    const int64_t head_bytes = g->block_size * g->head_dim * g->dtype_bytes;
+    const int64_t l0 = g->dec_pp_rank * Ld, l1 = l0 + Ld;
+    const int64_t h0 = g->dec_tp_rank * Hd, h1 = h0 + Hd;
+    const int64_t src_block = Lc * Hc * head_bytes, dst_block = Ld * Hd * head_bytes;
+    if (src_block >= (1ll << 32) || dst_block >= (1ll << 32))
+        return fail(KVM_EINVAL, "a block of %lld bytes is beyond the 4 GiB this kernel addresses",
+                    (long long)std::max(src_block, dst_block));
+
+    plan->segs.clear();
+    plan->dst_block_stride = (uint64_t)dst_block;
+    plan->payload_per_block = 2 * dst_block;
+    plan->min_src_blocks = INT64_MAX;
+    uint64_t align_bits = (uint64_t)head_bytes | (uint64_t)(uintptr_t)dst_k | (uint64_t)(uintptr_t)dst_v;
+
+    std::lock_guard<std::mutex> lock(g_mu);
+    for (int64_t p = l0 / Lc; p * Lc < l1; ++p) {
+        for (int64_t t = h0 / Hc; t * Hc < h1; ++t) {
+            auto it = g_sources.find({(int32_t)p, (int32_t)t});
+            if (it == g_sources.end())
+                return fail(KVM_ENOTREG, "context rank (pp %lld, tp %lld) is not registered",
+                            (long long)p, (long long)t);
+            const Source &src = it->second;
+            if (src.ctx_pp_size != g->ctx_pp_size || src.ctx_tp_size != g->ctx_tp_size ||
+                src.num_layers != g->num_layers || src.num_kv_heads != g->num_kv_heads)
+                return fail(KVM_EMISMATCH,
+                            "context rank (pp %lld, tp %lld) was registered for pp %d tp %d L %lld H %lld, "
+                            "call says pp %d tp %d L %lld H %lld",
+                            (long long)p, (long long)t, src.ctx_pp_size, src.ctx_tp_size,
+                            (long long)src.num_layers, (long long)src.num_kv_heads, g->ctx_pp_size,
+                            g->ctx_tp_size, (long long)g->num_layers, (long long)g->num_kv_heads);
+            if (src.nbytes % src_block)
+                return fail(KVM_EMISMATCH,
+                            "context pool (pp %lld, tp %lld) of %lld bytes is not a whole number of %lld-byte blocks",
+                            (long long)p, (long long)t, (long long)src.nbytes, (long long)src_block);
+            plan->min_src_blocks = std::min(plan->min_src_blocks, src.nbytes / src_block);
+
+            const int64_t la = std::max(l0, p * Lc), lb = std::min(l1, (p + 1) * Lc);
+            const int64_t ha = std::max(h0, t * Hc), hb = std::min(h1, (t + 1) * Hc);
+            const int64_t src_off = ((la - p * Lc) * Hc + (ha - t * Hc)) * head_bytes;
+            Seg s{};
+            s.src_k = src.k + src_off;
+            s.src_v = src.v + src_off;
+            s.src_block_stride = (uint64_t)src_block;
+            s.src_row_stride = (uint32_t)(Hc * head_bytes);
+            s.dst_row_stride = (uint32_t)(Hd * head_bytes);
+            s.dst_off = (uint32_t)(((la - l0) * Hd + (ha - h0)) * head_bytes);
+            s.run_bytes = (uint32_t)((hb - ha) * head_bytes);
+            s.n_rows = (uint32_t)(lb - la);
+            collapse(s);
+            plan->segs.push_back(s);
+            align_bits |= (uint64_t)(uintptr_t)src.k | (uint64_t)(uintptr_t)src.v;
+        }
+    }
+    plan->vec = vec_width(align_bits);
+    return KVM_OK;
+}
+
+// Enqueues the copy kernel over `segs` x `pairs`, as many launches as the 4 KiB argument needs.
+int launch_copy(std::vector<Seg> segs, const IdxPair *pairs, int64_t n, char *dst_k, char *dst_v,
+                uint64_t dst_block_stride, int vec, hipStream_t stream, int64_t *out_launches,
+                int64_t *out_wgs_per_block, int *out_threads)
+{
+    const Launch k = pick_kernel(vec);
+    uint32_t tile_bytes = (uint32_t)opt_tile_bytes.load();
+    int64_t launches = 0, wgs_per_block = 0;
+    for (size_t s0 = 0; s0 < segs.size(); s0 += kMaxSegs) {
+        MigrateArgs args;
+        args.dst_k = dst_k;
+        args.dst_v = dst_v;
+        args.dst_block_stride = dst_block_stride;
+        args.nseg = (uint32_t)std::min<size_t>(kMaxSegs, segs.size() - s0);
+        uint32_t tiles_total = 0;
+        for (uint32_t j = 0; j < args.nseg; ++j) {
+            Seg s = segs[s0 + j];
+            uint32_t tiles = 0;
+            tile_segment(s, tile_bytes, &tiles);
+            tiles_total += tiles;
+            s.tile_end = tiles_total;
+            args.seg[j] = s;
+        }
+        wgs_per_block += 2 * (int64_t)tiles_total;
+        for (int64_t i0 = 0; i0 < n; i0 += kMaxIdx) {
+            args.nidx = (uint32_t)std::min<int64_t>(kMaxIdx, n - i0);
+            if (pairs) {
+                memcpy(args.idx, pairs + i0, args.nidx * sizeof(IdxPair));
+                hipLaunchKernelGGL(k.fn, dim3(tiles_total, args.nidx, 2), dim3(k.threads), 0, stream, args);
+                KVM_HIP(hipGetLastError());
+            }
+            ++launches;
+        }
+        if (n == 0) ++launches;
+    }
+    if (out_launches) *out_launches = launches;
+    if (out_wgs_per_block) *out_wgs_per_block = wgs_per_block;
+    if (out_threads) *out_threads = k.threads;
+    return KVM_OK;
+}
+
+// dec index list must not repeat: the copies of one call run concurrently.
+thread_local std::vector<uint64_t> g_seen;
+
+int check_indices(const int64_t *src, const int64_t *dst, int64_t n, int64_t n_src, int64_t n_dst,
+                  const char *src_name, const char *dst_name, std::vector<IdxPair> *pairs)
+{
+    if (n_dst > INT32_MAX || n_src > INT32_MAX)
+        return fail(KVM_EINVAL, "pools of more than 2^31 blocks are not supported");
+    g_seen.assign((size_t)((n_dst + 63) / 64), 0);
+    pairs->resize((size_t)n);
+    for (int64_t i = 0; i < n; ++i) {
+        const int64_t a = src[i], b = dst[i];
+        if (a < 0 || a >= n_src)
+            return fail(KVM_ERANGE, "%s[%lld] = %lld is outside [0, %lld)", src_name, (long long)i,
+                        (long long)a, (long long)n_src);
+        if (b < 0 || b >= n_dst)
+            return fail(KVM_ERANGE, "%s[%lld] = %lld is outside [0, %lld)", dst_name, (long long)i,
+                        (long long)b, (long long)n_dst);
+        uint64_t &w = g_seen[(size_t)(b >> 6)];
+        const uint64_t bit = 1ull << (b & 63);
+        if (w & bit)
+            return fail(KVM_EDUP, "%s names block %lld twice", dst_name, (long long)b);
+        w |= bit;
+        (*pairs)[(size_t)i] = IdxPair{(int32_t)a, (int32_t)b};
+    }
+    return KVM_OK;
+}
+
+int device_of(const void *p, const char *what, int *device)
+{
+    hipPointerAttribute_t at;
+    hipError_t e = hipPointerGetAttributes(&at, p);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        return fail(KVM_EINVAL, "%s (%p) is not memory HIP knows: %s", what, p, hipGetErrorString(e));
+    }
+    if (at.type != hipMemoryTypeDevice)
+        return fail(KVM_EINVAL, "%s (%p) is not device memory", what, p);
+    *device = at.device;
+    return KVM_OK;
+}
+
+int host_pinned(const void *p, const char *what)
+{
+    hipPointerAttribute_t at;
+    hipError_t e = hipPointerGetAttributes(&at, p);
+    if (e != hipSuccess || at.type != hipMemoryTypeHost) {
+        (void)hipGetLastError();
+        return fail(KVM_EINVAL, "%s (%p) is not pinned host memory", what, p);
+    }
+    return KVM_OK;
+}
+
+// Pointers already checked by device_of / host_pinned (the query costs microseconds).
+std::mutex g_checked_mu;
+std::map<const void *, int> g_checked;  // ptr -> device, or -1 for pinned host
+
+int checked_device(const void *p, const char *what)
+{
+    {
+        std::lock_guard<std::mutex> lock(g_checked_mu);
+        auto it = g_checked.find(p);
+        if (it != g_checked.end() && it->second >= 0) return KVM_OK;
+    }
+    int dev = 0;
+    if (int rc = device_of(p, what, &dev)) return rc;
+    std::lock_guard<std::mutex> lock(g_checked_mu);
+    if (g_checked.size() > 64) g_checked.clear();
+    g_checked[p] = dev;
+    return KVM_OK;
+}
+
+int checked_pinned(const void *p, const char *what)
+{
+    {
+        std::lock_guard<std::mutex> lock(g_checked_mu);
+        auto it = g_checked.find(p);
+        if (it != g_checked.end() && it->second == -1) return KVM_OK;
+    }
+    if (int rc = host_pinned(p, what)) return rc;
+    std::lock_guard<std::mutex> lock(g_checked_mu);
+    if (g_checked.size() > 64) g_checked.clear();
+    g_checked[p] = -1;
+    return KVM_OK;
+}
+
+}  // namespace
+
+// ------------------------------------------------------------------------- C ABI
+
+extern "C" {
+
+int kvm_version(void) { return 100; }
+
+const char *kvm_last_error(void) { return g_err.c_str(); }
+
+int kvm_set_option(const char *name, int64_t value)
+{
+    std::atomic<int64_t> *o = find_opt(name);
+    if (!o) return fail(KVM_EINVAL, "unknown option '%s'", name ? name : "(null)");
+    bool ok = true;
+    if (o == &opt_tile_bytes) ok = value >= 4096 && value <= (1 << 26) && (value & (value - 1)) == 0;
+    else if (o == &opt_threads) ok = value == 256 || value == 512 || value == 1024;
+    else if (o == &opt_unroll) ok = value == 1 || value == 2 || value == 4 || value == 8;
+    else ok = value == 0 || value == 1;
+    if (!ok) return fail(KVM_EINVAL, "value %lld is not valid for option '%s'", (long long)value, name);
+    o->store(value);
+    return KVM_OK;
+}
+
+int64_t kvm_get_option(const char *name)
+{
+    std::atomic<int64_t> *o = find_opt(name);
+    if (!o) return fail(KVM_EINVAL, "unknown option '%s'", name ? name : "(null)");
+    return o->load();
+}
+
+int kvm_get_mem_handle(const void *dev_ptr, int64_t nbytes, int64_t *out_handle)
+{
+    if (!dev_ptr || !out_handle || nbytes <= 0)
+        return fail(KVM_EINVAL, "kvm_get_mem_handle: null pointer or non-positive size");
+    int dev = 0;
+    if (int rc = device_of(dev_ptr, "pool", &dev)) return rc;
+    memset(out_handle, 0, sizeof(int64_t) * KVM_HANDLE_WORDS);
+    out_handle[0] = kHandleMagic;
+    out_handle[1] = (int64_t)getpid();
+    out_handle[2] = dev;
+    out_handle[3] = (int64_t)(uintptr_t)dev_ptr;
+    out_handle[4] = nbytes;
+    out_handle[5] = out_handle[0] ^ out_handle[1] ^ out_handle[2] ^ out_handle[3] ^ out_handle[4];
+    return KVM_OK;
+}
+
+static int open_handle(const int64_t *h, const char *what, const char **ptr, int64_t *nbytes)
+{
+    if (!h) return fail(KVM_EINVAL, "%s handle is null", what);
+    if (h[0] != kHandleMagic || h[5] != (h[0] ^ h[1] ^ h[2] ^ h[3] ^ h[4]))
+        return fail(KVM_EHANDLE, "%s handle is not a kvmove memory handle", what);
+    if (h[1] != (int64_t)getpid())
+        return fail(KVM_EHANDLE,
+                    "%s handle was made by process %lld; this build resolves handles inside one process only",
+                    what, (long long)h[1]);
+    *ptr = (const char *)(uintptr_t)h[3];
+    *nbytes = h[4];
+    return KVM_OK;
+}
+
+int kvm_register_source(int32_t ctx_pp_size, int32_t ctx_tp_size, int32_t pp_rank, int32_t tp_rank,
+                        int64_t num_layers, int64_t num_kv_heads, const void *k_base,
+                        const void *v_base, int64_t nbytes_each)
+{
+    if (!k_base || !v_base || nbytes_each <= 0)
+        return fail(KVM_EINVAL, "kvm_register_source: null pool or non-positive size");
+    if (ctx_pp_size <= 0 || ctx_tp_size <= 0 || pp_rank < 0 || pp_rank >= ctx_pp_size || tp_rank < 0 ||
+        tp_rank >= ctx_tp_size)
+        return fail(KVM_EINVAL, "context rank (pp %d, tp %d) outside (pp %d, tp %d)", pp_rank, tp_rank,
+                    ctx_pp_size, ctx_tp_size);
+    if (num_layers <= 0 || num_kv_heads <= 0 || num_layers % ctx_pp_size || num_kv_heads % ctx_tp_size)
+        return fail(KVM_EINVAL, "L %lld / H %lld do not split over pp %d / tp %d", (long long)num_layers,
+                    (long long)num_kv_heads, ctx_pp_size, ctx_tp_size);
+    int dk = 0, dv = 0;
+    if (int rc = device_of(k_base, "context K pool", &dk)) return rc;
+    if (int rc = device_of(v_base, "context V pool", &dv)) return rc;
+    if (dk != dv) return fail(KVM_EINVAL, "context K and V pools sit on different devices");
+    Source s{ctx_pp_size, ctx_tp_size, num_layers, num_kv_heads, (const char *)k_base,
+             (const char *)v_base, nbytes_each};
+    std::lock_guard<std::mutex> lock(g_mu);
+    g_sources[{pp_rank, tp_rank}] = s;
+    return KVM_OK;
+}
+
+int kvm_register_mem_handle(const int64_t *k_handle, const int64_t *v_handle, int64_t num_layers,
+                            int64_t num_kv_heads, const int64_t context_pc[4],
+                            const int64_t decoding_pc[4])
+{
+    if (!context_pc || !decoding_pc) return fail(KVM_EINVAL, "parallel config list is null");
+    const char *k = nullptr, *v = nullptr;
+    int64_t kb = 0, vb = 0;
+    if (int rc = open_handle(k_handle, "K", &k, &kb)) return rc;
+    if (int rc = open_handle(v_handle, "V", &v, &vb)) return rc;
+    if (kb != vb) return fail(KVM_EMISMATCH, "K pool (%lld bytes) and V pool (%lld bytes) differ",
+                              (long long)kb, (long long)vb);
+    // [tp_size, tp_rank, pp_size, pp_rank]; the decoding list only has to be well formed here,
+    // the decoding rank's rectangle is taken from each migrate call.
+    if (decoding_pc[0] <= 0 || decoding_pc[2] <= 0 || decoding_pc[1] < 0 || decoding_pc[1] >= decoding_pc[0] ||
+        decoding_pc[3] < 0 || decoding_pc[3] >= decoding_pc[2])
+        return fail(KVM_EINVAL, "decoding parallel config [%lld,%lld,%lld,%lld] is malformed",
+                    (long long)decoding_pc[0], (long long)decoding_pc[1], (long long)decoding_pc[2],
+                    (long long)decoding_pc[3]);
+    return kvm_register_source((int32_t)context_pc[2], (int32_t)context_pc[0], (int32_t)context_pc[3],
+                               (int32_t)context_pc[1], num_layers, num_kv_heads, k, v, kb);
+}
+
+int kvm_reset(void)
+{
+    std::lock_guard<std::mutex> lock(g_mu);
+    g_sources.clear();
+    std::lock_guard<std::mutex> lock2(g_checked_mu);
+    g_checked.clear();
+    return KVM_OK;
+}
+
+int kvm_migrate_plan(const KvmGeom *geom, int64_t n, const void *dst_k, const void *dst_v, int64_t out[6])
+{
+    if (!out) return fail(KVM_EINVAL, "out is null");
+    Plan plan;
+    if (int rc = build_plan(geom, dst_k, dst_v, &plan)) return rc;
+    int64_t launches = 0, wgs = 0;
+    int threads = 0;
+    if (int rc = launch_copy(plan.segs, nullptr, n, nullptr, nullptr, plan.dst_block_stride, plan.vec,
+                             nullptr, &launches, &wgs, &threads))
+        return rc;
+    out[0] = wgs;
+    out[1] = threads;
+    out[2] = plan.vec;
+    out[3] = (int64_t)plan.segs.size();
+    out[4] = launches;
+    out[5] = plan.payload_per_block;
+    return KVM_OK;
+}
+
+int kvm_migrate(const KvmGeom *geom, const int64_t *ctx_idx, const int64_t *dec_idx, int64_t n,
+                void *dst_k, void *dst_v, int64_t dst_num_blocks, void *stream)
+{
+    if (n < 0) return fail(KVM_EINVAL, "n is negative");
+    if (!dst_k || !dst_v) return fail(KVM_EINVAL, "destination pool is null");
+    if (dst_num_blocks <= 0) return fail(KVM_EINVAL, "destination pool has no blocks");
+    if (n > 0 && (!ctx_idx || !dec_idx)) return fail(KVM_EINVAL, "index list is null");
+    Plan plan;
+    if (int rc = build_plan(geom, dst_k, dst_v, &plan)) return rc;
+    if (int rc = checked_device(dst_k, "decoding K pool")) return rc;
+    if (int rc = checked_device(dst_v, "decoding V pool")) return rc;
+    if (n == 0) return KVM_OK;
+    std::vector<IdxPair> pairs;
+    if (int rc = check_indices(ctx_idx, dec_idx, n, plan.min_src_blocks, dst_num_blocks,
+                               "context_block_indexes", "decoding_block_indexes", &pairs))
+        return rc;
+    return launch_copy(std::move(plan.segs), pairs.data(), n, (char *)dst_k, (char *)dst_v,
+                       plan.dst_block_stride, plan.vec, (hipStream_t)stream, nullptr, nullptr, nullptr);
+}
+
+int kvm_swap(const int64_t *src_ids, const int64_t *dst_ids, int64_t n, int is_swap_in, void *k_gpu,
+             void *v_gpu, void *k_host, void *v_host, int64_t slab_bytes, int64_t n_gpu_blocks,
+             int64_t n_host_blocks, void *stream)
+{
+    if (n < 0) return fail(KVM_EINVAL, "n is negative");
+    if (!k_gpu || !v_gpu || !k_host || !v_host) return fail(KVM_EINVAL, "a pool pointer is null");
+    if (slab_bytes <= 0 || slab_bytes >= (1ll << 32))
+        return fail(KVM_EINVAL, "slab_bytes %lld must be in (0, 4 GiB)", (long long)slab_bytes);
+    if (n_gpu_blocks <= 0 || n_host_blocks <= 0) return fail(KVM_EINVAL, "a pool has no blocks");
+    if (n > 0 && (!src_ids || !dst_ids)) return fail(KVM_EINVAL, "index list is null");
+    if (int rc = checked_device(k_gpu, "GPU K pool")) return rc;
+    if (int rc = checked_device(v_gpu, "GPU V pool")) return rc;
+    if (int rc = checked_pinned(k_host, "host K pool")) return rc;
+    if (int rc = checked_pinned(v_host, "host V pool")) return rc;
+    if (n == 0) return KVM_OK;
+
+    const int64_t n_src = is_swap_in ? n_host_blocks : n_gpu_blocks;
+    const int64_t n_dst = is_swap_in ? n_gpu_blocks : n_host_blocks;
+    std::vector<IdxPair> pairs;
+    if (int rc = check_indices(src_ids, dst_ids, n, n_src, n_dst, "source_block_ids", "target_block_ids",
+                               &pairs))
+        return rc;
+    char *src_k = (char *)(is_swap_in ? k_host : k_gpu), *src_v = (char *)(is_swap_in ? v_host : v_gpu);
+    char *dst_k = (char *)(is_swap_in ? k_gpu : k_host), *dst_v = (char *)(is_swap_in ? v_gpu : v_host);
+    hipStream_t st = (hipStream_t)stream;
+
+    if (opt_swap_mode.load() == 1) {
+        // One gather launch; the pinned pools are read or written in place over the host link.
+        void *dk = nullptr, *dv = nullptr;
+        KVM_HIP(hipHostGetDevicePointer(&dk, k_host, 0));
+        KVM_HIP(hipHostGetDevicePointer(&dv, v_host, 0));
+        if (is_swap_in) { src_k = (char *)dk; src_v = (char *)dv; }
+        else { dst_k = (char *)dk; dst_v = (char *)dv; }
+        Seg s{};
+        s.src_k = src_k;
+        s.src_v = src_v;
+        s.src_block_stride = (uint64_t)slab_bytes;
+        s.src_row_stride = s.dst_row_stride = s.run_bytes = (uint32_t)slab_bytes;
+        s.n_rows = 1;
+        const int vec = vec_width((uint64_t)slab_bytes | (uintptr_t)src_k | (uintptr_t)src_v |
+                                  (uintptr_t)dst_k | (uintptr_t)dst_v);
+        return launch_copy({s}, pairs.data(), n, dst_k, dst_v, (uint64_t)slab_bytes, vec, st, nullptr,
+                           nullptr, nullptr);
+    }
+
+    // hipMemcpyAsync per run of blocks that are consecutive on both sides.
+    const hipMemcpyKind kind = is_swap_in ? hipMemcpyHostToDevice : hipMemcpyDeviceToHost;
+    int64_t i = 0;
+    while (i < n) {
+        int64_t j = i + 1;
+        while (j < n && pairs[j].ctx == pairs[j - 1].ctx + 1 && pairs[j].dec == pairs[j - 1].dec + 1) ++j;
+        const size_t bytes = (size_t)(j - i) * (size_t)slab_bytes;
+        const size_t so = (size_t)pairs[i].ctx * (size_t)slab_bytes;
+        const size_t dof = (size_t)pairs[i].dec * (size_t)slab_bytes;
+        KVM_HIP(hipMemcpyAsync(dst_k + dof, src_k + so, bytes, kind, st));
+        KVM_HIP(hipMemcpyAsync(dst_v + dof, src_v + so, bytes, kind, st));
+        i = j;
+    }
+    return KVM_OK;
+}
+
+int kvm_copy_plain(void *dst, const void *src, int64_t nbytes, void *stream)
+{
+    if (!dst || !src || nbytes < 0) return fail(KVM_EINVAL, "kvm_copy_plain: null pointer or negative size");
+    if (nbytes == 0) return KVM_OK;
+    // Expressed as one segment over 4 MiB "blocks" with identity index pairs; K and V
+    // stand for the two halves of the buffer so that both grid planes do work.
+    const int64_t chunk = 4ll << 20;
+    const int64_t half_chunks = nbytes / (2 * chunk);
+    const int vec = vec_width((uint64_t)(uintptr_t)dst | (uint64_t)(uintptr_t)src | (uint64_t)nbytes);
+    int64_t done = 0;
+    if (half_chunks > 0) {
+        Seg s{};
+        s.src_k = (const char *)src;
+        s.src_v = (const char *)src + half_chunks * chunk;
+        s.src_block_stride = (uint64_t)chunk;
+        s.src_row_stride = s.dst_row_stride = s.run_bytes = (uint32_t)chunk;
+        s.n_rows = 1;
+        std::vector<IdxPair> pairs((size_t)half_chunks);
+        for (int64_t i = 0; i < half_chunks; ++i) pairs[(size_t)i] = IdxPair{(int32_t)i, (int32_t)i};
+        if (int rc = launch_copy({s}, pairs.data(), half_chunks, (char *)dst,
+                                 (char *)dst + half_chunks * chunk, (uint64_t)chunk, vec,
+                                 (hipStream_t)stream, nullptr, nullptr, nullptr))
+            return rc;
+        done = 2 * half_chunks * chunk;
+    }
+    if (done < nbytes)
+        KVM_HIP(hipMemcpyAsync((char *)dst + done, (const char *)src + done, (size_t)(nbytes - done),
+                               hipMemcpyDeviceToDevice, (hipStream_t)stream));
+    return KVM_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,131 @@
+"""Block-table handoff between the context (prefill) instance and the decoding instance.
+
+In-process mirror of the parts of reference ``distserve/single_stage_engine.py`` that sit
+on the KV movement path: pool set-up and handle exchange (``_init_kvcache`` :194-223,
+``register_kvcache_mem_handles`` :469-483), the tail of the context step that turns a
+prefilled request into a ``MigratingRequest`` (:393-401), ``_migrate_blocks`` (:490-536)
+and ``clear_migrated_blocks_callback`` (:405-410).  Scheduling, batching, the model
+forward and the Ray/asyncio plumbing are not part of this path: workers are plain
+objects on one GPU and a "remote call" is a direct method call on every worker.
+"""
+from __future__ import annotations
+
+import time
+from typing import Callable, Dict, List, Optional, Tuple
+
+from distserve_amd.block_manager import BlockManager
+from distserve_amd.config import CacheConfig, ModelConfig, ParallelConfig
+from distserve_amd.request import MigratingRequest, Request
+from distserve_amd.utils import MemoryHandle, Stage
+from distserve_amd.worker import Worker
+
+
+class SingleStageLLMEngine:
+    """What both instances share: a [pp][tp] grid of workers and one block manager."""
+
+    stage: Stage = None
+
+    def __init__(self, model_config: ModelConfig, parallel_config: ParallelConfig, cache_config: CacheConfig,
+                 worker_factory: Callable[..., Worker] = Worker):
+        self.model_config = model_config
+        self.parallel_config = parallel_config
+        self.cache_config = cache_config
+        self.workers: List[List[Worker]] = []
+        for pp_rank in range(parallel_config.pipeline_parallel_size):
+            row = []
+            for tp_rank in range(parallel_config.tensor_parallel_size):
+                rank_config = ParallelConfig(parallel_config.tensor_parallel_size, tp_rank,
+                                             parallel_config.pipeline_parallel_size, pp_rank)
+                worker_id = pp_rank * parallel_config.tensor_parallel_size + tp_rank
+                row.append(worker_factory(worker_id, self.stage, model_config, cache_config, rank_config))
+            self.workers.append(row)
+        self.kv_cache_mem_handles: List[List[Tuple[MemoryHandle, MemoryHandle]]] = []
+        self.block_manager: Optional[BlockManager] = None
+
+    def _remote_call_all_workers_async(self, func_name: str, *args) -> list:
+        """Call ``func_name`` on every worker, pipeline stage by stage (reference :225-233)."""
+        return [getattr(worker, func_name)(*args) for row in self.workers for worker in row]
+
+    def _init_kvcache(self, num_gpu_blocks: int, num_cpu_blocks: int) -> Tuple[int, int]:
+        """Allocate every worker's pools and collect the handles as ``[pp][tp]``."""
+        if self.stage == Stage.CONTEXT:
+            num_cpu_blocks = 1   # the context instance never swaps (reference :206-209)
+        flat = self._remote_call_all_workers_async("init_kvcache_and_swap", num_gpu_blocks, num_cpu_blocks)
+        tp = self.parallel_config.tensor_parallel_size
+        self.kv_cache_mem_handles = [flat[i:i + tp] for i in range(0, len(flat), tp)]
+        self.block_manager = BlockManager(self.stage, num_gpu_blocks, num_cpu_blocks, self.model_config,
+                                          self.parallel_config, self.cache_config,
+                                          self._remote_call_all_workers_async)
+        return num_gpu_blocks, num_cpu_blocks
+
+    def _free_request_resources(self, request_id: int) -> None:
+        self.block_manager.free_blocks(request_id)
+        self._remote_call_all_workers_async("clear_request_resource", request_id)
+
+
+class ContextStageLLMEngine(SingleStageLLMEngine):
+    stage = Stage.CONTEXT
+
+    def __init__(self, *args, **kwargs):
+        super().__init__(*args, **kwargs)
+        self.bridge_queue: List[MigratingRequest] = []
+
+    def on_prefill_finished(self, request: Request) -> MigratingRequest:
+        """Tail of the context step: the request's blocks stay where they are and their
+        table travels to the decoding instance (reference :393-401)."""
+        migrating_req = MigratingRequest(request, self.block_manager.get_block_table(request.request_id),
+                                         self.parallel_config)
+        self.bridge_queue.append(migrating_req)
+        return migrating_req
+
+    def clear_migrated_blocks_callback(self, migrated_request: MigratingRequest, migrate_events=()) -> None:
+        """Release the source blocks (reference :405-410).  Work the context workers enqueue
+        afterwards is ordered behind the migrations that read those blocks."""
+        for event in migrate_events:
+            self._remote_call_all_workers_async("wait_stream_for_migration", event)
+        self._free_request_resources(migrated_request.req.request_id)
+
+
+class DecodingStageLLMEngine(SingleStageLLMEngine):
+    stage = Stage.DECODING
+
+    def __init__(self, *args, clear_migrated_blocks_callback: Optional[Callable] = None, **kwargs):
+        super().__init__(*args, **kwargs)
+        self.clear_migrated_blocks_callback = clear_migrated_blocks_callback
+        self.lifetime_events: Dict[int, List[Tuple[str, float]]] = {}
+
+    def register_kvcache_mem_handles(self, context_parallel_config: ParallelConfig,
+                                     kv_cache_mem_handles: List[List[Tuple[MemoryHandle, MemoryHandle]]]) -> None:
+        """Hand the context instance's handles to every decoding worker (reference :469-483)."""
+        self.kv_cache_mem_handles = kv_cache_mem_handles
+        self._remote_call_all_workers_async("register_kvcache_mem_handles", context_parallel_config,
+                                            kv_cache_mem_handles)
+
+    def _migrate_blocks(self, migrating_req: MigratingRequest) -> None:
+        """Move one request from the context instance to this one (reference :490-536):
+        allocate blocks for its *prompt* here, have every decoding rank pull its share,
+        then release the blocks on the context side."""
+        req = migrating_req.req
+        # the first generated token already exists; it must not count towards the blocks
+        # that are allocated (and copied) now
+        kept = (req.generated_tokens, req.generated_token_ids)
+        req.generated_tokens, req.generated_token_ids = [], []
+        try:
+            self.block_manager.allocate_blocks(req)
+        finally:
+            req.generated_tokens, req.generated_token_ids = kept
+
+        target_block_indexes = self.block_manager.get_block_table(req.request_id)
+        assert len(target_block_indexes) == len(migrating_req.block_indexes), (
+            f"request {req.request_id}: {len(migrating_req.block_indexes)} context blocks but "
+            f"{len(target_block_indexes)} decoding blocks")
+
+        self.lifetime_events.setdefault(req.request_id, []).append(("migration_begin", time.time()))
+        self._remote_call_all_workers_async("migrate_blocks", migrating_req.block_indexes,
+                                            migrating_req.context_parallel_config, target_block_indexes)
+        self.lifetime_events[req.request_id].append(("migration_end", time.time()))
+
+        if self.clear_migrated_blocks_callback is not None:
+            events = [w.latest_migrate_event for row in self.workers for w in row
+                      if getattr(w, "latest_migrate_event", None) is not None]
+            self.clear_migrated_blocks_callback(migrating_req, events)

@@ -1,0 +1,158 @@
+/*
+ * kvmove -- C ABI of the MI355X (gfx950) KV-block migration and swap library.
+ *
+ * This is the drop-in boundary for the prefill->decode KV movement path of DistServe.
+ * Each entry point names the reference call it stands behind (paths relative to the
+ * DistServe tree).  In the reference those calls go to SwiftTransformer's
+ * torch.ops.block_migration_ops.* / torch.ops.swapping_ops.swap (libst_pybinding.so);
+ * here a thin torch op shim with the same schemas (distserve_amd/csrc/kvmove_torch.cpp)
+ * forwards to these functions.
+ *
+ * Conventions
+ *   - plain pointers and sizes only; no C++ or torch types cross this boundary;
+ *   - every function returns KVM_OK (0) or a negative KVM_E* code and never throws;
+ *     kvm_last_error() returns the calling thread's last error text;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream); work is
+ *     enqueued on it and the call returns without waiting for the GPU;
+ *   - index arrays are read before the call returns (the caller may free them);
+ *   - pools are borrowed: the caller keeps them alive while work is in flight;
+ *   - calls may come from several host threads and target several streams.
+ *
+ * Pool layout (distserve/worker.py:107-121): contiguous
+ *     [num_blocks, layers_local, kv_heads_local, block_size, head_dim]
+ * K and V are separate pools of identical shape.  Pipeline rank p of P owns layers
+ * [p*L/P, (p+1)*L/P) (distserve/config.py:279-286); tensor rank t of T owns KV heads
+ * [t*H/T, (t+1)*H/T) (distserve/config.py:225-257).
+ */
+#ifndef KVMOVE_H
+#define KVMOVE_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define KVM_OK 0
+#define KVM_EINVAL (-1)     /* malformed argument (null pointer, bad size, bad geometry) */
+#define KVM_ERANGE (-2)     /* a block index is outside its pool */
+#define KVM_EDUP (-3)       /* a destination block index occurs twice in one call */
+#define KVM_ENOTREG (-4)    /* a context rank the copy needs was never registered */
+#define KVM_EHIP (-5)       /* a HIP runtime call failed */
+#define KVM_EHANDLE (-6)    /* memory handle is not one of this process's */
+#define KVM_EMISMATCH (-7)  /* registered pools disagree with the call's geometry */
+
+#define KVM_HANDLE_WORDS 8  /* int64 words in a memory handle */
+
+/* Whole-model KV geometry and both instances' layouts for one migrate call.
+ * The [tp_size, tp_rank, pp_size, pp_rank] order of ParallelConfig.to_list()
+ * (distserve/config.py:57-63) is unpacked into named fields here. */
+typedef struct KvmGeom {
+    int64_t num_layers;    /* L: layers of the whole model (ModelConfig.get_num_layers()) */
+    int64_t num_kv_heads;  /* H: KV heads of the whole model (ModelConfig.get_num_heads()) */
+    int64_t block_size;    /* B: tokens per block (CacheConfig.block_size) */
+    int64_t head_dim;      /* D */
+    int64_t dtype_bytes;   /* s: 2 for fp16, 4 for fp32 (ModelConfig.get_dtype_size()) */
+    int32_t ctx_pp_size;   /* context instance pipeline_parallel_size */
+    int32_t ctx_tp_size;   /* context instance tensor_parallel_size */
+    int32_t dec_pp_size;   /* decoding instance sizes ... */
+    int32_t dec_tp_size;
+    int32_t dec_pp_rank;   /* ... and the decoding rank that pulls */
+    int32_t dec_tp_rank;
+} KvmGeom;
+
+/* Library version: major*10000 + minor*100 + patch. */
+int kvm_version(void);
+
+/* Text of the last error on the calling thread ("" if none). */
+const char *kvm_last_error(void);
+
+/*
+ * Replaces torch.ops.block_migration_ops.get_ipc_mem_handle(tensor)
+ * (distserve/worker.py:133-134).  Writes an opaque KVM_HANDLE_WORDS-word token naming
+ * the device allocation [dev_ptr, dev_ptr + nbytes).  Single-GPU build: the token is
+ * valid only inside the process that made it (same-process pointer registry); a token
+ * from another process is refused with KVM_EHANDLE.
+ */
+int kvm_get_mem_handle(const void *dev_ptr, int64_t nbytes, int64_t *out_handle);
+
+/*
+ * Replaces torch.ops.block_migration_ops.register_ipc_mem_handle(k_handle, v_handle,
+ * num_layers, num_heads, context_parallel_config, decoding_parallel_config)
+ * (distserve/worker.py:239-246).  Binds context rank (pp_rank, tp_rank)'s K and V pools.
+ * context_pc / decoding_pc are [tp_size, tp_rank, pp_size, pp_rank]
+ * (distserve/config.py:57-63).  Registering the same rank again replaces the binding.
+ */
+int kvm_register_mem_handle(const int64_t *k_handle, const int64_t *v_handle,
+                            int64_t num_layers, int64_t num_kv_heads,
+                            const int64_t context_pc[4], const int64_t decoding_pc[4]);
+
+/* Same binding from raw device pointers (no handle round trip). */
+int kvm_register_source(int32_t ctx_pp_size, int32_t ctx_tp_size, int32_t pp_rank, int32_t tp_rank,
+                        int64_t num_layers, int64_t num_kv_heads,
+                        const void *k_base, const void *v_base, int64_t nbytes_each);
+
+/* Forget every registered context pool (the reference has no counterpart: its
+ * registry lives as long as the worker process; tests and benches need a clean slate). */
+int kvm_reset(void);
+
+/*
+ * Replaces torch.ops.block_migration_ops.migrate_blocks(...)
+ * (distserve/worker.py:250-267).  For i in [0, n), X in {K, V} and every (layer l,
+ * kv head h) of decoding rank (dec_pp_rank, dec_tp_rank):
+ *     dstX[dec_idx[i], l - l0_dec, h - h0_dec, :, :] =
+ *         srcX{owner(l,h)}[ctx_idx[i], l - l0_ctx, h - h0_ctx, :, :]
+ * Source pools are the registered ones; they are only read.  Destination blocks not
+ * named in dec_idx are not touched.  dec_idx must not repeat a block (KVM_EDUP);
+ * ctx_idx may.  n == 0 is a no-op.
+ */
+int kvm_migrate(const KvmGeom *geom, const int64_t *ctx_idx, const int64_t *dec_idx, int64_t n,
+                void *dst_k, void *dst_v, int64_t dst_num_blocks, void *stream);
+
+/*
+ * Replaces torch.ops.swapping_ops.swap(source_block_ids, target_block_ids, is_swap_in,
+ * k_cache, v_cache, k_swap, v_swap) (distserve/worker.py:303-311).
+ * is_swap_in != 0:  gpuX[dst_ids[i]]  = hostX[src_ids[i]]
+ * is_swap_in == 0:  hostX[dst_ids[i]] = gpuX[src_ids[i]]        for X in {K, V}.
+ * slab_bytes is one block of one pool (layers_local*heads_local*B*D*s).  Host pools
+ * must be pinned (hipHostMalloc / torch pin_memory) for the copy to be asynchronous.
+ * dst_ids must not repeat a block.
+ */
+int kvm_swap(const int64_t *src_ids, const int64_t *dst_ids, int64_t n, int is_swap_in,
+             void *k_gpu, void *v_gpu, void *k_host, void *v_host, int64_t slab_bytes,
+             int64_t n_gpu_blocks, int64_t n_host_blocks, void *stream);
+
+/*
+ * Plain contiguous device copy with the same load/store code as the migration kernel.
+ * No counterpart in the reference: it calibrates hardware counters (a copy of known
+ * size) and gives the attainable streaming-copy ceiling beside the migration figure.
+ */
+int kvm_copy_plain(void *dst, const void *src, int64_t nbytes, void *stream);
+
+/*
+ * Tuning knobs (no counterpart in the reference).  Names:
+ *   "tile_bytes"     payload bytes one workgroup moves per pool kind (power of two >= 4096)
+ *   "threads"        workgroup size: 256, 512 or 1024
+ *   "unroll"         16-byte vectors in flight per lane: 1, 2, 4 or 8
+ *   "nt_load"        1 = nontemporal loads, 0 = plain
+ *   "nt_store"       1 = nontemporal stores, 0 = plain
+ *   "swap_mode"      0 = hipMemcpyAsync per contiguous run, 1 = copy kernel over pinned memory
+ * kvm_get_option returns the value or KVM_EINVAL (as int64) for an unknown name.
+ */
+int kvm_set_option(const char *name, int64_t value);
+int64_t kvm_get_option(const char *name);
+
+/*
+ * Launch shape kvm_migrate would use for this geometry and n blocks, for tests and
+ * reports: out[0] = workgroups per block (K and V together), out[1] = workgroup size,
+ * out[2] = vector width in bytes, out[3] = number of source segments,
+ * out[4] = kernel launches, out[5] = payload bytes per block (K+V, this rank's share).
+ * Needs the sources registered (alignment of their bases picks the vector width).
+ */
+int kvm_migrate_plan(const KvmGeom *geom, int64_t n, const void *dst_k, const void *dst_v,
+                     int64_t out[6]);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* KVMOVE_H */

@@ -1,0 +1,81 @@
+"""The C-ABI library loads, exports every symbol include/kvmove.h declares and refuses
+malformed arguments without touching a GPU."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "kvmove.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(kvm_\w+)\s*\(", text)))
+
+
+def test_every_declared_symbol_is_exported(kvm):
+    names = declared_symbols()
+    assert len(names) >= 12 and set(names) == set(kvm.EXPORTS)
+    raw = ctypes.CDLL(os.path.join(ROOT, "distserve_amd", "lib", "libkvmove.so"))
+    for name in names:
+        assert getattr(raw, name) is not None
+
+
+def test_version_and_options(kvm):
+    assert kvm.version() >= 100
+    assert kvm.get_option("tile_bytes") >= 4096
+    old = kvm.get_option("unroll")
+    kvm.set_option("unroll", 8)
+    assert kvm.get_option("unroll") == 8
+    kvm.set_option("unroll", old)
+    for name, bad in (("tile_bytes", 5000), ("threads", 128), ("unroll", 3), ("nt_store", 2), ("nope", 1)):
+        with pytest.raises(kvm.KvmError) as e:
+            kvm.set_option(name, bad)
+        assert e.value.code == kvm.KVM_EINVAL
+
+
+def test_argument_errors_need_no_gpu(kvm, fresh_registry):
+    g = kvm.geom(4, 4, 16, 8, 2)
+    with pytest.raises(kvm.KvmError) as e:
+        kvm.migrate(g, [0], [0], 0, 0, 4)                       # null destination
+    assert e.value.code == kvm.KVM_EINVAL
+    bad = kvm.geom(5, 4, 16, 8, 2, ctx_pp=2)                    # 5 layers over pp 2
+    with pytest.raises(kvm.KvmError) as e:
+        kvm.migrate(bad, [0], [0], 4096, 8192, 4)
+    assert e.value.code == kvm.KVM_EINVAL and "divisible" in str(e.value)
+    with pytest.raises(kvm.KvmError) as e:
+        kvm.migrate(kvm.geom(4, 4, 16, 8, 2, dec_tp=2, dec_tp_rank=2), [0], [0], 4096, 8192, 4)
+    assert e.value.code == kvm.KVM_EINVAL
+    with pytest.raises(kvm.KvmError) as e:
+        kvm.migrate(g, [0], [0], 4096, 8192, 4)                 # nothing registered
+    assert e.value.code == kvm.KVM_ENOTREG
+    with pytest.raises(kvm.KvmError) as e:
+        kvm.register_mem_handle([0] * 8, [0] * 8, 4, 4, [1, 0, 1, 0], [1, 0, 1, 0])
+    assert e.value.code == kvm.KVM_EHANDLE
+    with pytest.raises(kvm.KvmError) as e:
+        kvm.swap([0], [0], True, 0, 0, 0, 0, 64, 1, 1)
+    assert e.value.code == kvm.KVM_EINVAL
+
+
+def test_torch_ops_are_registered_with_the_reference_argument_order():
+    import torch
+
+    import distserve_amd  # noqa: F401  (loads the shim)
+
+    s = str(torch.ops.block_migration_ops.migrate_blocks.default._schema)
+    order = ["context_pp_size", "context_tp_size", "context_block_indexes", "decoding_pp_size", "decoding_tp_size",
+             "decoding_pp_rank", "decoding_tp_rank", "decoding_block_indexes", "k_cache", "v_cache"]
+    assert [s.index(a) for a in order] == sorted(s.index(a) for a in order)
+    s = str(torch.ops.swapping_ops.swap.default._schema)
+    order = ["source_block_ids", "target_block_ids", "is_swap_in", "k_cache", "v_cache", "k_swap", "v_swap"]
+    assert [s.index(a) for a in order] == sorted(s.index(a) for a in order)
+    s = str(torch.ops.block_migration_ops.register_ipc_mem_handle.default._schema)
+    order = ["k_handle", "v_handle", "num_layers", "num_heads", "context_parallel_config", "decoding_parallel_config"]
+    assert [s.index(a) for a in order] == sorted(s.index(a) for a in order)
+    assert "int[]" in str(torch.ops.block_migration_ops.get_ipc_mem_handle.default._schema)
+    # no CPU fallback: a CPU tensor is refused, loudly
+    z = torch.zeros(2, 1, 1, 2, 2, dtype=torch.float16)
+    with pytest.raises(RuntimeError, match="GPU"):
+        torch.ops.block_migration_ops.migrate_blocks(1, 1, [0], 1, 1, 0, 0, [0], z, z)

@@ -1,0 +1,105 @@
+"""The migration handoff protocol with fake workers (no GPU): order of the steps, the
+fan-out to every decoding rank and the block tables that travel (reference
+distserve/single_stage_engine.py:393-410, 469-536)."""
+import pytest
+
+from distserve_amd.config import CacheConfig, ModelConfig, ParallelConfig
+from distserve_amd.handoff import ContextStageLLMEngine, DecodingStageLLMEngine
+from distserve_amd.request import create_request
+
+LOG = []
+
+
+class FakeWorker:
+    def __init__(self, worker_id, stage, model_config, cache_config, parallel_config):
+        self.worker_id, self.stage, self.parallel_config = worker_id, stage, parallel_config
+        self.latest_migrate_event = None
+
+    def _tag(self):
+        return (str(self.stage), self.parallel_config.pipeline_parallel_rank, self.parallel_config.tensor_parallel_rank)
+
+    def init_kvcache_and_swap(self, n_gpu, n_cpu):
+        LOG.append(("init",) + self._tag() + (n_gpu, n_cpu))
+        return ([1, self.worker_id], [2, self.worker_id])
+
+    def register_kvcache_mem_handles(self, ctx_pc, handles):
+        LOG.append(("register",) + self._tag() + (ctx_pc.to_list(), handles))
+
+    def migrate_blocks(self, ctx_idx, ctx_pc, dec_idx):
+        LOG.append(("migrate",) + self._tag() + (list(ctx_idx), ctx_pc.to_list(), list(dec_idx)))
+        self.latest_migrate_event = ("event", self.worker_id)
+
+    def wait_stream_for_migration(self, event):
+        LOG.append(("wait",) + self._tag() + (event,))
+
+    def clear_request_resource(self, request_id):
+        LOG.append(("clear",) + self._tag() + (request_id,))
+
+
+@pytest.fixture()
+def engines():
+    LOG.clear()
+    model = ModelConfig.from_kv_shape(8, 8, 16)
+    cache = CacheConfig(16, 128)
+    ctx = ContextStageLLMEngine(model, ParallelConfig(2, 0, 2, 0), cache, worker_factory=FakeWorker)
+    dec = DecodingStageLLMEngine(model, ParallelConfig(4, 0, 1, 0), cache, worker_factory=FakeWorker,
+                                 clear_migrated_blocks_callback=ctx.clear_migrated_blocks_callback)
+    ctx._init_kvcache(10, 7)
+    dec._init_kvcache(12, 5)
+    return ctx, dec
+
+
+def test_init_collects_handles_as_pp_by_tp_and_context_never_swaps(engines):
+    ctx, dec = engines
+    inits = [e for e in LOG if e[0] == "init"]
+    assert [e[1:4] for e in inits[:4]] == [("context", 0, 0), ("context", 0, 1), ("context", 1, 0), ("context", 1, 1)]
+    assert all(e[4:] == (10, 1) for e in inits[:4])          # num_cpu_blocks forced to 1
+    assert all(e[4:] == (12, 5) for e in inits[4:])
+    assert ctx.kv_cache_mem_handles == [[([1, 0], [2, 0]), ([1, 1], [2, 1])], [([1, 2], [2, 2]), ([1, 3], [2, 3])]]
+    dec.register_kvcache_mem_handles(ctx.parallel_config, ctx.kv_cache_mem_handles)
+    regs = [e for e in LOG if e[0] == "register"]
+    assert [e[2:4] for e in regs] == [(0, 0), (0, 1), (0, 2), (0, 3)]     # every decoding rank
+    assert all(e[5] == ctx.kv_cache_mem_handles for e in regs)
+
+
+def test_migrate_allocates_prompt_blocks_fans_out_then_frees_the_source(engines):
+    ctx, dec = engines
+    LOG.clear()
+    warm = create_request(16, 90)
+    ctx.block_manager.allocate_blocks(warm)                       # context block 0 is taken
+    req = create_request(40, 7)                                   # 3 blocks
+    ctx.block_manager.allocate_blocks(req)                        # context blocks [1,2,3]
+    req.add_generated_token("t", 5)                               # prefill produced the first token
+    for _ in range(8):
+        req.add_generated_token("t", 5)                           # 49 tokens would be 4 blocks
+    m = ctx.on_prefill_finished(req)
+    assert m.block_indexes == [1, 2, 3] and ctx.bridge_queue == [m]
+
+    dec._migrate_blocks(m)
+    # the generated tokens came back and did not size the allocation
+    assert req.get_output_len() == 9
+    assert dec.block_manager.get_block_table(7) == [0, 1, 2]
+    migrates = [e for e in LOG if e[0] == "migrate"]
+    assert [(e[2], e[3]) for e in migrates] == [(0, 0), (0, 1), (0, 2), (0, 3)]
+    for e in migrates:
+        assert e[4] == [1, 2, 3] and e[5] == [2, 0, 2, 0] and e[6] == [0, 1, 2]
+    # order: all migrations, then the context workers wait on their events, then the free
+    kinds = [e[0] for e in LOG]
+    assert kinds.index("wait") > max(i for i, k in enumerate(kinds) if k == "migrate")
+    assert kinds.index("clear") > max(i for i, k in enumerate(kinds) if k == "wait")
+    assert len([k for k in kinds if k == "wait"]) == 4 * 4          # 4 events x 4 context workers
+    assert 7 not in ctx.block_manager.block_table
+    assert ctx.block_manager.free_gpu_blocks_list[-3:] == [1, 2, 3]
+    assert [n for n, _ in dec.lifetime_events[7]] == ["migration_begin", "migration_end"]
+
+
+def test_length_mismatch_is_refused_before_any_copy(engines):
+    ctx, dec = engines
+    req = create_request(40, 3)
+    ctx.block_manager.allocate_blocks(req)
+    m = ctx.on_prefill_finished(req)
+    m.block_indexes = m.block_indexes[:-1]
+    LOG.clear()
+    with pytest.raises(AssertionError):
+        dec._migrate_blocks(m)
+    assert not [e for e in LOG if e[0] == "migrate"]
