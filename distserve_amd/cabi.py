@@ -84,7 +84,14 @@ def _check(rc: int) -> None:
 
 
 def _arr(values: Sequence[int]):
+    if isinstance(values, ctypes.Array):
+        return values
     return (ctypes.c_int64 * len(values))(*values)
+
+
+def index_array(values: Sequence[int]):
+    """A block-index list converted once, for callers that reuse it across calls."""
+    return _arr(list(values))
 
 
 def version() -> int:

@@ -1,0 +1,254 @@
+"""Parity of the HIP migration path against the CPU oracle, called through the C ABI.
+Bit-exact: pools are compared as raw 16/32-bit patterns."""
+import itertools
+import json
+import os
+
+import pytest
+import torch
+
+import oracle
+from distserve_amd import workloads
+from gpu_helpers import gpu_migrate, kvm_geom, oracle_migrate, stream_handle, upload_and_register
+from helpers import canary_pool, geom_of, make_src_pools, same_bits
+
+pytestmark = pytest.mark.gpu
+
+
+def check_case(kvm, g, nb_src, nb_dst, ci, di, seed=1, dtype=torch.float16):
+    kvm.reset()
+    src_k = make_src_pools(g, nb_src, seed, dtype)
+    src_v = make_src_pools(g, nb_src, seed + 500, dtype)
+    keep = upload_and_register(g, src_k, src_v)
+    got_k, got_v = gpu_migrate(g, ci, di, nb_dst, dtype)
+    want_k, want_v = oracle_migrate(g, src_k, src_v, ci, di, nb_dst, dtype)
+    assert same_bits(got_k, want_k), "K pool differs from the oracle"
+    assert same_bits(got_v, want_v), "V pool differs from the oracle"
+    # sources are only read
+    for p in range(g.ctx_pp):
+        for t in range(g.ctx_tp):
+            assert same_bits(keep[0][p][t].cpu(), src_k[p][t]) and same_bits(keep[1][p][t].cpu(), src_v[p][t])
+    kvm.reset()
+
+
+def test_config1_gpt2_small_bit_exact(kvm):
+    w = workloads.config1()
+    call = w.calls[0]
+    check_case(kvm, geom_of(w), w.src_blocks, w.dst_blocks, call.ctx_idx, call.dec_idx, seed=w.seed)
+
+
+@pytest.mark.parametrize("cpp,ctp,dpp,dtp", list(itertools.product((1, 2, 4), repeat=4)))
+def test_every_layout_and_every_decoding_rank(kvm, cpp, ctp, dpp, dtp):
+    ci, di = [3, 0, 4, 3], [1, 5, 2, 0]
+    for q in range(dpp):
+        for u in range(dtp):
+            g = oracle.Geom(4, 4, 16, 8, 2, cpp, ctp, dpp, dtp, q, u)
+            check_case(kvm, g, 5, 6, ci, di, seed=7)
+
+
+def test_golden_fixtures(kvm):
+    import hashlib
+    from golden.make_golden import build_case
+
+    path = os.path.join(os.path.dirname(__file__), "golden", "migrate_golden.json")
+    for case in json.load(open(path))["cases"]:
+        kvm.reset()
+        g, src_k, src_v, ci, di, nb_dst = build_case(case)
+        keep = upload_and_register(g, src_k, src_v)
+        got_k, got_v = gpu_migrate(g, ci, di, nb_dst)
+        for kind, got in (("k", got_k), ("v", got_v)):
+            digest = hashlib.sha256(oracle.bits(got.contiguous()).numpy().tobytes()).hexdigest()
+            assert digest == case["sha256_" + kind], (case["name"], kind)
+        del keep
+    kvm.reset()
+
+
+@pytest.mark.parametrize("B,D,s,dtype", [(16, 128, 2, torch.float16), (16, 64, 4, torch.float32),
+                                         (1, 4, 2, torch.float16), (3, 5, 2, torch.float16),
+                                         (1, 1, 2, torch.float16), (7, 3, 4, torch.float32)])
+def test_block_and_head_sizes_down_to_narrow_vectors(kvm, B, D, s, dtype):
+    """Head slabs of 4 KiB down to 2 bytes: the vector width falls from 16 bytes to 2."""
+    g = oracle.Geom(4, 6, B, D, s, 2, 3, 1, 2, 0, 1)
+    check_case(kvm, g, 9, 11, [8, 2, 0, 5, 7], [10, 0, 3, 6, 1], seed=13, dtype=dtype)
+    kvm.reset()
+
+
+def test_misaligned_pool_bases_pick_a_narrower_vector(kvm):
+    g = oracle.Geom(2, 2, 4, 8, 2)                      # 64-byte head slabs
+    kvm.reset()
+    src_k = make_src_pools(g, 6, 3)[0][0]
+    src_v = make_src_pools(g, 6, 4)[0][0]
+    n = src_k.numel()
+    raw_k = torch.zeros(n + 8, dtype=torch.float16, device="cuda")
+    raw_v = torch.zeros(n + 8, dtype=torch.float16, device="cuda")
+    dk, dv = raw_k[2:2 + n], raw_v[2:2 + n]             # bases 4 bytes past a 16-byte boundary
+    dk.copy_(src_k.flatten())
+    dv.copy_(src_v.flatten())
+    kvm.register_source(1, 1, 0, 0, 2, 2, dk.data_ptr(), dv.data_ptr(), n * 2)
+    dst_k = canary_pool(g.dec_pool_shape(5)).cuda()
+    dst_v = canary_pool(g.dec_pool_shape(5)).cuda()
+    plan = kvm.migrate_plan(kvm_geom(g), 3, dst_k.data_ptr(), dst_v.data_ptr())
+    assert plan["vector_bytes"] == 4
+    kvm.migrate(kvm_geom(g), [5, 0, 2], [1, 4, 0], dst_k.data_ptr(), dst_v.data_ptr(), 5, stream_handle())
+    torch.cuda.synchronize()
+    want_k, want_v = oracle_migrate(g, [[src_k]], [[src_v]], [5, 0, 2], [1, 4, 0], 5)
+    assert same_bits(dst_k.cpu(), want_k) and same_bits(dst_v.cpu(), want_v)
+    kvm.reset()
+
+
+@pytest.mark.parametrize("n", [0, 1, 439, 440, 441, 881, 1000])
+def test_list_lengths_around_the_per_launch_limit(kvm, n):
+    """One launch carries 440 index pairs; longer lists split into several launches."""
+    g = oracle.Geom(2, 2, 16, 8, 2)
+    gen = torch.Generator().manual_seed(n)
+    ci = torch.randint(0, 64, (n,), generator=gen).tolist()          # context blocks may repeat
+    di = torch.randperm(1200, generator=gen)[:n].tolist()
+    check_case(kvm, g, 64, 1200, ci, di, seed=5)
+
+
+def test_more_context_ranks_than_one_launch_holds(kvm):
+    """pp4 x tp4 context ranks all feed one decoding rank: 16 segments, 8 per launch."""
+    g = oracle.Geom(8, 8, 16, 8, 2, 4, 4, 1, 1, 0, 0)
+    check_case(kvm, g, 7, 9, [6, 1, 3], [0, 8, 4], seed=17)
+    kvm.reset()
+    keep = upload_and_register(g, make_src_pools(g, 7, 1), make_src_pools(g, 7, 2))
+    dst = canary_pool(g.dec_pool_shape(9)).cuda()
+    plan = kvm.migrate_plan(kvm_geom(g), 3, dst.data_ptr(), dst.data_ptr())
+    assert plan["segments"] == 16 and plan["launches"] == 2
+    del keep
+    kvm.reset()
+
+
+@pytest.mark.parametrize("tile_bytes,threads,unroll", [(4096, 256, 1), (8192, 512, 2), (32768, 256, 4),
+                                                       (65536, 1024, 8), (1 << 20, 512, 8), (16384, 1024, 4)])
+def test_every_tuning_choice_copies_the_same_bytes(kvm, tile_bytes, threads, unroll):
+    saved = {k: kvm.get_option(k) for k in ("tile_bytes", "threads", "unroll", "nt_load", "nt_store")}
+    try:
+        kvm.set_option("tile_bytes", tile_bytes)
+        kvm.set_option("threads", threads)
+        kvm.set_option("unroll", unroll)
+        for ntl, nts in ((1, 1), (0, 0)):
+            kvm.set_option("nt_load", ntl)
+            kvm.set_option("nt_store", nts)
+            # 24 KiB rows (cfg1 shape), 80 KiB rows (TP2->1) and 8 KiB strided rows (GQA slice)
+            check_case(kvm, oracle.Geom(3, 12, 16, 64, 2), 6, 7, [5, 1, 2], [0, 6, 3], seed=3)
+            check_case(kvm, oracle.Geom(4, 40, 16, 128, 2, 1, 2, 1, 1), 4, 5, [3, 1], [0, 4], seed=4)
+            check_case(kvm, oracle.Geom(12, 8, 16, 128, 2, 2, 2, 1, 4, 0, 1), 5, 6, [4, 0, 2], [1, 5, 3], seed=5)
+    finally:
+        for k, v in saved.items():
+            kvm.set_option(k, v)
+
+
+def test_errors_leave_the_destination_untouched(kvm):
+    g = oracle.Geom(2, 4, 16, 8, 2, 1, 2, 1, 1)
+    kvm.reset()
+    src_k, src_v = make_src_pools(g, 4, 1), make_src_pools(g, 4, 2)
+    keep = upload_and_register(g, src_k, src_v)
+    dst_k = canary_pool(g.dec_pool_shape(6)).cuda()
+    dst_v = canary_pool(g.dec_pool_shape(6)).cuda()
+    args = (dst_k.data_ptr(), dst_v.data_ptr(), 6, stream_handle())
+    cases = [
+        ([0, 1], [2, 2], kvm.KVM_EDUP),             # decoding block named twice
+        ([4], [0], kvm.KVM_ERANGE),                 # context index == pool size
+        ([-1], [0], kvm.KVM_ERANGE),
+        ([0], [6], kvm.KVM_ERANGE),
+        ([0], [-3], kvm.KVM_ERANGE),
+        ([0, 1], [0], kvm.KVM_EINVAL),              # lists of different length
+    ]
+    for ci, di, code in cases:
+        with pytest.raises(kvm.KvmError) as e:
+            kvm.migrate(kvm_geom(g), ci, di, *args)
+        assert e.value.code == code, (ci, di, str(e.value))
+    # geometry that disagrees with what was registered
+    with pytest.raises(kvm.KvmError) as e:
+        kvm.migrate(kvm_geom(oracle.Geom(2, 4, 16, 8, 2, 1, 1, 1, 1)), [0], [0], *args)
+    assert e.value.code in (kvm.KVM_EMISMATCH, kvm.KVM_ENOTREG)
+    # a geometry whose blocks do not tile the registered pools
+    with pytest.raises(kvm.KvmError) as e:
+        kvm.migrate(kvm_geom(oracle.Geom(2, 4, 16, 24, 2, 1, 2, 1, 1)), [0], [0], *args)
+    assert e.value.code == kvm.KVM_EMISMATCH
+    # a host pointer is not a pool
+    host = torch.zeros(1024, dtype=torch.float16)
+    with pytest.raises(kvm.KvmError) as e:
+        kvm.migrate(kvm_geom(g), [0], [0], host.data_ptr(), host.data_ptr(), 1, stream_handle())
+    assert e.value.code == kvm.KVM_EINVAL
+    torch.cuda.synchronize()
+    assert same_bits(dst_k.cpu(), canary_pool(g.dec_pool_shape(6)))
+    assert same_bits(dst_v.cpu(), canary_pool(g.dec_pool_shape(6)))
+    del keep
+    kvm.reset()
+
+
+@pytest.mark.parametrize("make,layers", [(workloads.config2, 2), (workloads.config3, 2), (workloads.config4, 4)])
+def test_configs_2_3_4_block_tables_on_a_thinner_model(kvm, make, layers):
+    """The measured configurations' real block tables, rank layouts, head counts and head
+    size on a model with fewer layers, so that the oracle finishes in seconds.  Calls that
+    recycle block ids are verified one by one."""
+    w = workloads.scaled(make(), num_layers=layers)
+    g = geom_of(w)
+    kvm.reset()
+    src_k = make_src_pools(g, w.src_blocks, w.seed)
+    src_v = make_src_pools(g, w.src_blocks, w.seed + 500)
+    keep = upload_and_register(g, src_k, src_v)
+    dst_k = canary_pool(g.dec_pool_shape(w.dst_blocks)).cuda()
+    dst_v = canary_pool(g.dec_pool_shape(w.dst_blocks)).cuda()
+    want_k = canary_pool(g.dec_pool_shape(w.dst_blocks))
+    want_v = canary_pool(g.dec_pool_shape(w.dst_blocks))
+    for call in w.calls:
+        kvm.migrate(kvm_geom(g), call.ctx_idx, call.dec_idx, dst_k.data_ptr(), dst_v.data_ptr(), w.dst_blocks,
+                    stream_handle())
+        oracle.migrate_c(g, src_k, call.ctx_idx, call.dec_idx, want_k)
+        oracle.migrate_c(g, src_v, call.ctx_idx, call.dec_idx, want_v)
+        if w.recycles_blocks:
+            torch.cuda.synchronize()
+            idx = torch.tensor(call.dec_idx)
+            assert same_bits(dst_k.cpu()[idx], want_k[idx]) and same_bits(dst_v.cpu()[idx], want_v[idx]), call.request_id
+    torch.cuda.synchronize()
+    assert same_bits(dst_k.cpu(), want_k) and same_bits(dst_v.cpu(), want_v)
+    del keep
+    kvm.reset()
+
+
+def test_config2_full_size_properties(kvm):
+    """LLaMA-2-7B shape at full size (two 32 GiB pool pairs): every migrated block equals its
+    source (checked on the GPU with torch's own gather), every other destination block
+    still holds the canary, and sampled blocks agree with the oracle on the CPU."""
+    w = workloads.config2()
+    g = geom_of(w)
+    kvm.reset()
+    shape_src, shape_dst = w.src_pool_shape(), w.dst_pool_shape()
+    src_k = workloads.fill_uniform(shape_src, w.seed, "cuda")
+    src_v = workloads.fill_uniform(shape_src, w.seed + 500, "cuda")
+    dst_k = workloads.fill_canary(shape_dst, "cuda")
+    dst_v = workloads.fill_canary(shape_dst, "cuda")
+    kvm.register_source(1, 1, 0, 0, g.num_layers, g.num_kv_heads, src_k.data_ptr(), src_v.data_ptr(),
+                        src_k.numel() * 2)
+    for call in w.calls:                                   # one call per request, as the engine does
+        kvm.migrate(kvm_geom(g), call.ctx_idx, call.dec_idx, dst_k.data_ptr(), dst_v.data_ptr(), w.dst_blocks,
+                    stream_handle())
+    torch.cuda.synchronize()
+    ctx = torch.tensor([b for c in w.calls for b in c.ctx_idx], device="cuda")
+    dec = torch.tensor([b for c in w.calls for b in c.dec_idx], device="cuda")
+    for src, dst in ((src_k, dst_k), (src_v, dst_v)):
+        for i0 in range(0, ctx.numel(), 128):
+            a = dst.view(torch.int16)[dec[i0:i0 + 128]]
+            b = src.view(torch.int16)[ctx[i0:i0 + 128]]
+            assert torch.equal(a, b)
+        untouched = torch.ones(w.dst_blocks, dtype=torch.bool, device="cuda")
+        untouched[dec] = False
+        rest = untouched.nonzero().flatten()
+        for i0 in range(0, rest.numel(), 256):
+            assert bool((dst.view(torch.int16)[rest[i0:i0 + 256]] == workloads.CANARY_BITS).all())
+    # oracle on a sample: compact the touched blocks into small CPU pools
+    pick = list(range(0, ctx.numel(), max(1, ctx.numel() // 24)))[:24]
+    ci = [int(ctx[i]) for i in pick]
+    di = [int(dec[i]) for i in pick]
+    small_src_k = src_k[torch.tensor(ci, device="cuda")].cpu()
+    small_src_v = src_v[torch.tensor(ci, device="cuda")].cpu()
+    want_k = canary_pool(g.dec_pool_shape(len(pick)))
+    want_v = canary_pool(g.dec_pool_shape(len(pick)))
+    oracle.migrate_c(g, [[small_src_k]], list(range(len(pick))), list(range(len(pick))), want_k)
+    oracle.migrate_c(g, [[small_src_v]], list(range(len(pick))), list(range(len(pick))), want_v)
+    assert same_bits(dst_k[torch.tensor(di, device="cuda")].cpu(), want_k)
+    assert same_bits(dst_v[torch.tensor(di, device="cuda")].cpu(), want_v)
+    kvm.reset()

@@ -1,0 +1,143 @@
+"""Parity of the swap path (HBM <-> pinned host) against the CPU oracle through the C ABI,
+in both implementations (hipMemcpyAsync per run, copy kernel over pinned memory), and
+its overlap with a migration on another stream."""
+import pytest
+import torch
+
+import oracle
+from distserve_amd import workloads
+from gpu_helpers import kvm_geom, upload_and_register
+from helpers import canary_pool, geom_of, make_src_pools, rand_pool, same_bits
+
+pytestmark = pytest.mark.gpu
+
+BLOCK = (3, 4, 16, 32)          # layers, heads, block_size, head_dim -> 12 KiB slabs
+
+
+@pytest.fixture(params=[0, 1], ids=["memcpy", "kernel"])
+def swap_mode(kvm, request):
+    old = kvm.get_option("swap_mode")
+    kvm.set_option("swap_mode", request.param)
+    yield request.param
+    kvm.set_option("swap_mode", old)
+
+
+def pools(n_gpu, n_host, seed, block=BLOCK):
+    k_gpu = rand_pool((n_gpu,) + block, seed).cuda()
+    v_gpu = rand_pool((n_gpu,) + block, seed + 1).cuda()
+    k_host = canary_pool((n_host,) + block).pin_memory()
+    v_host = canary_pool((n_host,) + block).pin_memory()
+    return k_gpu, v_gpu, k_host, v_host
+
+
+def do_swap(kvm, src, dst, swap_in, k_gpu, v_gpu, k_host, v_host, stream=None):
+    slab = k_gpu[0].numel() * k_gpu.element_size()
+    s = (stream or torch.cuda.current_stream()).cuda_stream
+    kvm.swap(src, dst, swap_in, k_gpu.data_ptr(), v_gpu.data_ptr(), k_host.data_ptr(), v_host.data_ptr(),
+             slab, k_gpu.shape[0], k_host.shape[0], s)
+
+
+def test_swap_out_then_in_matches_oracle_and_round_trips(kvm, swap_mode):
+    k_gpu, v_gpu, k_host, v_host = pools(12, 9, seed=3)
+    k0, v0 = k_gpu.cpu(), v_gpu.cpu()
+    out_src, out_dst = [7, 0, 1, 2, 11, 5], [3, 8, 4, 5, 0, 6]        # holds a run 0,1,2 -> 4,5 (partly)
+    do_swap(kvm, out_src, out_dst, False, k_gpu, v_gpu, k_host, v_host)
+    torch.cuda.synchronize()
+    want_k, want_v = canary_pool(k_host.shape), canary_pool(v_host.shape)
+    oracle.swap_c(out_src, out_dst, k0, want_k)
+    oracle.swap_c(out_src, out_dst, v0, want_v)
+    assert same_bits(k_host, want_k) and same_bits(v_host, want_v)
+    assert same_bits(k_gpu.cpu(), k0) and same_bits(v_gpu.cpu(), v0)       # swap-out only reads HBM
+
+    in_dst = [4, 9, 10, 3, 6, 8]                                         # other slots than they left
+    do_swap(kvm, out_dst, in_dst, True, k_gpu, v_gpu, k_host, v_host)
+    torch.cuda.synchronize()
+    exp_k, exp_v = k0.clone(), v0.clone()
+    oracle.swap_c(out_dst, in_dst, want_k, exp_k)
+    oracle.swap_c(out_dst, in_dst, want_v, exp_v)
+    assert same_bits(k_gpu.cpu(), exp_k) and same_bits(v_gpu.cpu(), exp_v)
+    for a, b in zip(out_src, in_dst):                                     # the round trip itself
+        assert same_bits(k_gpu[b].cpu(), k0[a]) and same_bits(v_gpu[b].cpu(), v0[a])
+
+
+def test_consecutive_ids_coalesce_without_changing_the_result(kvm, swap_mode):
+    k_gpu, v_gpu, k_host, v_host = pools(16, 16, seed=5)
+    k0 = k_gpu.cpu()
+    src = list(range(2, 12)) + [15, 0]
+    dst = list(range(4, 14)) + [1, 15]
+    do_swap(kvm, src, dst, False, k_gpu, v_gpu, k_host, v_host)
+    torch.cuda.synchronize()
+    want = canary_pool(k_host.shape)
+    oracle.swap_lib(src, dst, k0, want)
+    assert same_bits(k_host, want)
+
+
+def test_empty_and_single_and_whole_pool(kvm, swap_mode):
+    k_gpu, v_gpu, k_host, v_host = pools(5, 5, seed=9)
+    do_swap(kvm, [], [], False, k_gpu, v_gpu, k_host, v_host)
+    torch.cuda.synchronize()
+    assert same_bits(k_host, canary_pool(k_host.shape))
+    do_swap(kvm, [4], [0], False, k_gpu, v_gpu, k_host, v_host)
+    do_swap(kvm, [0, 1, 2, 3], [1, 2, 3, 4], False, k_gpu, v_gpu, k_host, v_host)
+    torch.cuda.synchronize()
+    assert same_bits(k_host[0], k_gpu[4].cpu())
+    assert same_bits(v_host[1:], v_gpu[:4].cpu())
+
+
+def test_swap_errors(kvm, swap_mode):
+    k_gpu, v_gpu, k_host, v_host = pools(4, 3, seed=1)
+    for src, dst, swap_in, code in [([4], [0], False, kvm.KVM_ERANGE), ([0], [3], False, kvm.KVM_ERANGE),
+                                    ([3], [0], True, kvm.KVM_ERANGE), ([0, 1], [2, 2], False, kvm.KVM_EDUP),
+                                    ([-1], [0], True, kvm.KVM_ERANGE)]:
+        with pytest.raises(kvm.KvmError) as e:
+            do_swap(kvm, src, dst, swap_in, k_gpu, v_gpu, k_host, v_host)
+        assert e.value.code == code
+    pageable = canary_pool(k_host.shape)                                   # not pinned: refused
+    with pytest.raises(kvm.KvmError) as e:
+        do_swap(kvm, [0], [0], False, k_gpu, v_gpu, pageable, v_host)
+    assert e.value.code == kvm.KVM_EINVAL and "pinned" in str(e.value)
+    torch.cuda.synchronize()
+    assert same_bits(k_host, canary_pool(k_host.shape))
+
+
+def test_config5_shape_swap_overlapping_a_migration(kvm, swap_mode):
+    """Configuration 5 on a thinner model (2 layers) and smaller pools: swap out, swap back
+    into other slots on side streams while a migration runs on the main stream."""
+    shape = workloads.KvShape(2, 32, 128)
+    w = workloads.config5(gpu_blocks=512, host_blocks=512, swap_blocks=256, migrate_requests=4,
+                          migrate_src_blocks=160, shape=shape, min_len=64, max_len=512)
+    g = geom_of(w.migrate)
+    kvm.reset()
+    block = shape.pool_shape(1)[1:]
+    k_gpu, v_gpu, k_host, v_host = pools(w.gpu_blocks, w.host_blocks, seed=w.seed, block=block)
+    k0, v0 = k_gpu.cpu(), v_gpu.cpu()
+    src_k, src_v = make_src_pools(g, w.migrate.src_blocks, 77), make_src_pools(g, w.migrate.src_blocks, 78)
+    keep = upload_and_register(g, src_k, src_v)
+    out_stream, in_stream = torch.cuda.Stream(), torch.cuda.Stream()
+    torch.cuda.synchronize()
+
+    do_swap(kvm, w.out_gpu_ids, w.out_host_ids, False, k_gpu, v_gpu, k_host, v_host, out_stream)
+    out_done = torch.cuda.Event()
+    out_done.record(out_stream)
+    for call in w.migrate.calls:                     # main stream, concurrent with the swaps
+        kvm.migrate(kvm_geom(g), call.ctx_idx, call.dec_idx, k_gpu.data_ptr(), v_gpu.data_ptr(), w.gpu_blocks,
+                    torch.cuda.current_stream().cuda_stream)
+    in_stream.wait_event(out_done)                   # swap-in reuses slots the swap-out frees
+    do_swap(kvm, w.out_host_ids, w.in_gpu_ids, True, k_gpu, v_gpu, k_host, v_host, in_stream)
+    torch.cuda.synchronize()
+
+    exp_k, exp_v = k0.clone(), v0.clone()
+    host_k, host_v = canary_pool(k_host.shape), canary_pool(v_host.shape)
+    oracle.swap_c(w.out_gpu_ids, w.out_host_ids, k0, host_k)
+    oracle.swap_c(w.out_gpu_ids, w.out_host_ids, v0, host_v)
+    oracle.swap_c(w.out_host_ids, w.in_gpu_ids, host_k, exp_k)
+    oracle.swap_c(w.out_host_ids, w.in_gpu_ids, host_v, exp_v)
+    for call in w.migrate.calls:
+        oracle.migrate_c(g, src_k, call.ctx_idx, call.dec_idx, exp_k)
+        oracle.migrate_c(g, src_v, call.ctx_idx, call.dec_idx, exp_v)
+    assert same_bits(k_host, host_k) and same_bits(v_host, host_v)
+    assert same_bits(k_gpu.cpu(), exp_k) and same_bits(v_gpu.cpu(), exp_v)
+    for a, b in zip(w.out_gpu_ids, w.in_gpu_ids):
+        assert a != b and same_bits(k_gpu[b].cpu(), k0[a])
+    del keep
+    kvm.reset()

@@ -1,0 +1,114 @@
+"""The drop-in surface end to end on the GPU: torch.ops schemas, Worker, BlockManager and
+the migration handoff, against the CPU oracle."""
+import pytest
+import torch
+
+import oracle
+import distserve_amd
+from distserve_amd import (BlockManager, CacheConfig, ContextStageLLMEngine, DecodingStageLLMEngine, ModelConfig,
+                           ParallelConfig, Worker, create_request)
+from distserve_amd.utils import Stage
+from helpers import canary_pool, rand_pool, same_bits
+
+pytestmark = pytest.mark.gpu
+
+
+def fill(worker, seed):
+    worker.k_cache.copy_(rand_pool(worker.k_cache.shape, seed))
+    worker.v_cache.copy_(rand_pool(worker.v_cache.shape, seed + 1))
+
+
+def test_ops_registered_and_refuse_cpu_tensors():
+    z = torch.zeros(2, 1, 1, 2, 2, dtype=torch.float16)
+    with pytest.raises(RuntimeError, match="GPU"):
+        torch.ops.block_migration_ops.migrate_blocks(1, 1, [0], 1, 1, 0, 0, [0], z, z)
+    with pytest.raises(RuntimeError):
+        torch.ops.block_migration_ops.get_ipc_mem_handle(z)
+
+
+def test_handoff_tp2pp2_to_tp4_every_rank_against_oracle(kvm):
+    """Context TP2/PP2 -> decoding TP4 (the layout of configuration 4) through Worker,
+    BlockManager and the handoff; every decoding rank's pools are checked."""
+    kvm.reset()
+    model = ModelConfig.from_kv_shape(num_layers=8, num_heads=32, head_dim=64, num_kv_heads=8)
+    cache = CacheConfig(16, 64)
+    ctx = ContextStageLLMEngine(model, ParallelConfig(2, 0, 2, 0), cache)
+    dec = DecodingStageLLMEngine(model, ParallelConfig(4, 0, 1, 0), cache,
+                                 clear_migrated_blocks_callback=ctx.clear_migrated_blocks_callback)
+    ctx._init_kvcache(24, 0)
+    dec._init_kvcache(32, 4)
+    dec.register_kvcache_mem_handles(ctx.parallel_config, ctx.kv_cache_mem_handles)
+    for i, w in enumerate(w for row in ctx.workers for w in row):
+        fill(w, 100 + 10 * i)
+    for w in dec.workers[0]:
+        w.k_cache.view(torch.int16).fill_(0x7C01)
+        w.v_cache.view(torch.int16).fill_(0x7C01)
+    src_k = [[w.k_cache.cpu() for w in row] for row in ctx.workers]
+    src_v = [[w.v_cache.cpu() for w in row] for row in ctx.workers]
+    want_k = [canary_pool(w.k_cache.shape) for w in dec.workers[0]]
+    want_v = [canary_pool(w.v_cache.shape) for w in dec.workers[0]]
+
+    # some context blocks are already in use, so the tables are not 0..n on both sides
+    ctx.block_manager.allocate_blocks(create_request(50, 900))
+    dec.block_manager.allocate_blocks(create_request(20, 901))
+    for rid, prompt_len in enumerate([40, 16, 97]):
+        req = create_request(prompt_len, rid)
+        ctx.block_manager.allocate_blocks(req)
+        req.add_generated_token("x", 1)
+        m = ctx.on_prefill_finished(req)
+        ci = list(m.block_indexes)
+        dec._migrate_blocks(m)
+        di = dec.block_manager.get_block_table(rid)
+        assert len(ci) == len(di) == -(-prompt_len // 16)
+        for u in range(4):
+            g = oracle.Geom(8, 8, 16, 64, 2, 2, 2, 1, 4, 0, u)
+            oracle.migrate_c(g, src_k, ci, di, want_k[u])
+            oracle.migrate_c(g, src_v, ci, di, want_v[u])
+        assert rid not in ctx.block_manager.block_table          # source blocks released
+    torch.cuda.synchronize()
+    for u, w in enumerate(dec.workers[0]):
+        assert same_bits(w.k_cache.cpu(), want_k[u]) and same_bits(w.v_cache.cpu(), want_v[u]), u
+    kvm.reset()
+
+
+def test_block_manager_swap_through_worker_round_trip(kvm):
+    kvm.reset()
+    model = ModelConfig.from_kv_shape(4, 8, 64)
+    cache = CacheConfig(16, 64)
+    worker = Worker(0, Stage.DECODING, model, cache)
+    worker.init_kvcache_and_swap(16, 12)
+    fill(worker, 5)
+    k0, v0 = worker.k_cache.cpu(), worker.v_cache.cpu()
+
+    def call_all(func_name, *args):
+        return [getattr(worker, func_name)(*args)]
+
+    bm = BlockManager(Stage.DECODING, 16, 12, model, ParallelConfig(), cache, call_all)
+    a, b = create_request(60, 0), create_request(33, 1)
+    bm.allocate_blocks(a)                                        # GPU [0..3]
+    bm.allocate_blocks(b)                                        # GPU [4,5,6]
+    bm.swap_out_requests([a, b])
+    assert bm.get_block_table(0) == [0, 1, 2, 3] and bm.get_location(0).value == "cpu"
+    filler = create_request(16 * 9, 2)
+    bm.allocate_blocks(filler)                                   # takes GPU [7..15]: free list is empty now
+    bm.swap_in_requests([b, a])                                  # must flush the swap-out quarantine
+    assert bm.get_block_table(1) == [0, 1, 2] and bm.get_block_table(0) == [3, 4, 5, 6]
+    worker.step([0, 1])                                          # compute stream waits for the swap-ins
+    torch.cuda.synchronize()
+    k1, v1 = worker.k_cache.cpu(), worker.v_cache.cpu()
+    assert same_bits(k1[0:3], k0[4:7]) and same_bits(v1[0:3], v0[4:7])       # request b
+    assert same_bits(k1[3:7], k0[0:4]) and same_bits(v1[3:7], v0[0:4])       # request a
+    assert same_bits(k1[7:], k0[7:])
+    assert worker.swap_event_table == {}
+    worker.wait_for_all_swap_in()
+    worker.wait_for_all_swap_out()
+    kvm.reset()
+
+
+def test_profile_and_block_bytes():
+    model = ModelConfig("meta-llama/Llama-2-7b-hf")
+    worker = Worker(0, Stage.DECODING, model, CacheConfig(16, 256, cpu_swap_space=2))
+    assert worker._get_block_size_in_bytes(16, model, ParallelConfig()) == 8 * 1024 * 1024
+    assert worker._get_block_size_in_bytes(16, model, ParallelConfig(2, 0, 2, 0)) == 2 * 1024 * 1024
+    n_gpu, n_cpu = worker._profile_num_available_blocks(16, 0.5, 2 << 30)
+    assert n_cpu == 256 and n_gpu > 1000
