@@ -41,7 +41,25 @@ def parse_args():
     ap.add_argument("--opt", action="append", default=[], help="kvmove tuning option name=value")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also time the plain contiguous copy kernel (adds launches to a profile)")
+    ap.add_argument("--plain-copy-only", type=int, default=0, metavar="MiB",
+                    help="launch nothing but plain contiguous copies of this size (counter calibration)")
     return ap.parse_args()
+
+
+def measured_traffic(config: int, algorithmic_bytes_per_launch: float):
+    """HBM bytes per launch from the committed hardware-counter summary of this configuration
+    (two rocprofv3 --pmc runs, FETCH_SIZE and WRITE_SIZE, each scaled by a plain copy of
+    known size), or None when no summary has been committed for it."""
+    import re
+
+    path = os.path.join(ROOT, "profiles", f"kvm_copy_kernel_cfg{config}_pmc.txt")
+    if not os.path.exists(path):
+        return None
+    m = re.search(r"TRAFFIC_PER_ALGORITHMIC_BYTE read=([0-9.]+) write=([0-9.]+)", open(path).read())
+    if not m:
+        return None
+    # algorithmic bytes are half reads and half writes
+    return round(algorithmic_bytes_per_launch * (float(m.group(1)) + float(m.group(2))) / 2)
 
 
 def make_calls(w, pattern):
@@ -129,6 +147,15 @@ def main():
     for kv in args.opt:
         name, value = kv.split("=")
         cabi.set_option(name, int(value))
+
+    if args.plain_copy_only:
+        torch.cuda.set_device(0)
+        nbytes = args.plain_copy_only << 20
+        gbps = time_plain_copy(cabi, torch.cuda.current_stream(), nbytes=nbytes, reps=args.steps, warm=args.warmup)
+        print(json.dumps({"metric": "plain contiguous copy", "value": gbps, "unit": "GB/s",
+                          "bytes_copied_per_call": nbytes, "hbm_bytes_per_call": 2 * nbytes,
+                          "launches_per_call": -(-(nbytes // (8 << 20)) // 440), "steps": args.steps}))
+        return
 
     if args.config == 5:
         from bench_swap import run_swap_bench
@@ -218,7 +245,7 @@ def main():
         "roofline": {
             "bound": "hbm", "achieved": round(bytes_per_launch / (launch_us * 1e-6) / 1e9, 2), "peak": HBM_PEAK_GBPS,
             "unit": "GB/s", "frac": round(bytes_per_launch / (launch_us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
-            "traffic": None,
+            "traffic": measured_traffic(args.config, bytes_per_launch),
             "kernel": "kvm_copy_kernel<u32x4>", "launches_per_step": launches_per_step,
             "avg_launch_us": round(launch_us, 2), "algorithmic_bytes_per_launch": round(bytes_per_launch),
             "workgroups_per_block": plan["workgroups_per_block"], "workgroup_size": plan["threads"],
@@ -267,13 +294,13 @@ def verify(w, src_k, src_v, dst_k, dst_v) -> bool:
     return ok
 
 
-def time_plain_copy(cabi, stream, nbytes=4 << 30, reps=10):
+def time_plain_copy(cabi, stream, nbytes=4 << 30, reps=10, warm=2):
     import torch
 
     a = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
     b = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
     a.fill_(3)
-    for _ in range(2):
+    for _ in range(warm):
         cabi.copy_plain(b.data_ptr(), a.data_ptr(), nbytes, stream.cuda_stream)
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     e0.record(stream)
