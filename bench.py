@@ -41,6 +41,9 @@ def parse_args():
     ap.add_argument("--opt", action="append", default=[], help="kvmove tuning option name=value")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also time the plain contiguous copy kernel (adds launches to a profile)")
+    ap.add_argument("--swap-blocks", type=int, default=0, help="config 5: blocks to swap (default 2048)")
+    ap.add_argument("--swap-wgs", type=int, nargs="*", default=[4],
+                    help="config 5: workgroup counts to try for the swap kernel")
     ap.add_argument("--plain-copy-only", type=int, default=0, metavar="MiB",
                     help="launch nothing but plain contiguous copies of this size (counter calibration)")
     return ap.parse_args()
@@ -158,8 +161,6 @@ def main():
         return
 
     if args.config == 5:
-        from bench_swap import run_swap_bench
-
         print(json.dumps(run_swap_bench(args)))
         return
 
@@ -258,6 +259,176 @@ def main():
         torch.cuda.empty_cache()
         out["cpu_baseline"] = cpu_baseline(w)
     print(json.dumps(out))
+
+
+def run_swap_bench(args):
+    """Configuration 5: swap 2048 blocks (16 GiB) from HBM to a pinned host pool and back into
+    other GPU slots, on side streams, while an 8-request migration runs on the main stream.
+    The denominator is the host link measured in the same run with one large pinned copy per
+    direction.  A step is one swap-out plus one swap-in of the whole block list."""
+    import torch
+
+    from distserve_amd import cabi, workloads
+
+    torch.cuda.set_device(0)
+    w = workloads.config5(swap_blocks=args.swap_blocks) if args.swap_blocks else workloads.config5()
+    shape = w.shape
+    main = torch.cuda.current_stream()
+    out_stream, in_stream = torch.cuda.Stream(), torch.cuda.Stream()
+
+    k_gpu = workloads.fill_uniform(shape.pool_shape(w.gpu_blocks), w.seed, "cuda")
+    v_gpu = workloads.fill_uniform(shape.pool_shape(w.gpu_blocks), w.seed + 500, "cuda")
+    k_ref, v_ref = k_gpu.clone(), v_gpu.clone()            # what the round trip must reproduce
+    t0 = time.perf_counter()
+    k_host = torch.empty(shape.pool_shape(w.host_blocks), dtype=shape.dtype, pin_memory=True)
+    v_host = torch.empty(shape.pool_shape(w.host_blocks), dtype=shape.dtype, pin_memory=True)
+    pin_s = time.perf_counter() - t0
+    mig = w.migrate
+    src_k = workloads.fill_uniform(mig.src_pool_shape(), 77, "cuda")
+    src_v = workloads.fill_uniform(mig.src_pool_shape(), 78, "cuda")
+    cabi.reset()
+    cabi.register_source(1, 1, 0, 0, shape.num_layers, shape.num_kv_heads, src_k.data_ptr(), src_v.data_ptr(),
+                         src_k.numel() * shape.dtype_bytes)
+    geom = cabi.geom(shape.num_layers, shape.num_kv_heads, shape.block_size, shape.head_dim, shape.dtype_bytes)
+    mig_calls = [(cabi.index_array(c.ctx_idx), cabi.index_array(c.dec_idx)) for c in mig.calls]
+    slab = w.slab_bytes
+    ptrs = (k_gpu.data_ptr(), v_gpu.data_ptr(), k_host.data_ptr(), v_host.data_ptr())
+    out_src, out_dst = cabi.index_array(w.out_gpu_ids), cabi.index_array(w.out_host_ids)
+    in_dst = cabi.index_array(w.in_gpu_ids)
+
+    # ---- the link itself: one large pinned copy per direction
+    link_bytes = 4 << 30
+    big_host = torch.empty(link_bytes, dtype=torch.uint8, pin_memory=True)
+    big_gpu = torch.empty(link_bytes, dtype=torch.uint8, device="cuda")
+
+    def timed(fn, stream):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        fn()
+        e1.record(stream)
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e-3
+
+    link = {}
+    for name, fn in (("d2h", lambda: big_host.copy_(big_gpu, non_blocking=True)),
+                     ("h2d", lambda: big_gpu.copy_(big_host, non_blocking=True))):
+        fn()
+        torch.cuda.synchronize()
+        link[name] = link_bytes / min(timed(fn, main) for _ in range(3)) / 1e9
+    del big_host, big_gpu
+
+    def migrate_once():
+        for ci, di in mig_calls:
+            cabi.migrate(geom, ci, di, k_gpu.data_ptr(), v_gpu.data_ptr(), w.gpu_blocks, main.cuda_stream)
+
+    def swap_out():
+        cabi.swap(out_src, out_dst, False, *ptrs, slab, w.gpu_blocks, w.host_blocks, out_stream.cuda_stream)
+
+    def swap_in():
+        cabi.swap(out_dst, in_dst, True, *ptrs, slab, w.gpu_blocks, w.host_blocks, in_stream.cuda_stream)
+
+    results = {}
+    bytes_dir = w.bytes_per_direction
+    default_mode, default_wgs = cabi.get_option("swap_mode"), cabi.get_option("swap_wgs")
+    if default_mode == 1 and default_wgs not in args.swap_wgs:
+        args.swap_wgs.append(default_wgs)
+
+    def migrate_timed():
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(main)
+        migrate_once()
+        e1.record(main)
+        return e0, e1
+
+    # touch every page of the pinned pools and warm both directions before anything is timed
+    swap_out()
+    in_stream.wait_stream(out_stream)
+    swap_in()
+    migrate_once()
+    torch.cuda.synchronize()
+    e0, e1 = migrate_timed()
+    torch.cuda.synchronize()
+    migrate_alone_ms = e0.elapsed_time(e1)
+
+    variants = [("hipMemcpyAsync per block", 0, None), ("hipMemcpyAsync per block, V on a forked stream", 2, None)]
+    variants += [(f"copy kernel over pinned memory, {g} workgroups per pool kind", 1, g) for g in args.swap_wgs]
+    for mode_name, mode, wgs in variants:
+        cabi.set_option("swap_mode", mode)
+        if wgs:
+            cabi.set_option("swap_wgs", wgs)
+        rows = []
+        for overlapped in (False, True):
+            k_gpu.copy_(k_ref)
+            v_gpu.copy_(v_ref)
+            torch.cuda.synchronize()
+            t_host = time.perf_counter()
+            e = [torch.cuda.Event(enable_timing=True) for _ in range(4)]
+            e[0].record(out_stream)
+            swap_out()
+            e[1].record(out_stream)
+            host_out_us = (time.perf_counter() - t_host) * 1e6
+            mig_ms = []
+            if overlapped:
+                m = [migrate_timed() for _ in range(3)]     # while the swap-out is in flight
+            in_stream.wait_event(e[1])        # swap-in reuses slots the swap-out frees
+            e[2].record(in_stream)
+            swap_in()
+            e[3].record(in_stream)
+            if overlapped:
+                main.wait_event(e[2])                       # start beside the swap-in
+                m += [migrate_timed() for _ in range(3)]
+            torch.cuda.synchronize()
+            if overlapped:
+                mig_ms = [round(a.elapsed_time(b), 3) for a, b in m]
+            t_out, t_in = e[0].elapsed_time(e[1]) * 1e-3, e[2].elapsed_time(e[3]) * 1e-3
+            ok = True
+            for ref, pool in ((k_ref, k_gpu), (v_ref, v_gpu)):
+                for i0 in range(0, len(w.out_gpu_ids), 256):
+                    a = torch.tensor(w.out_gpu_ids[i0:i0 + 256], device="cuda")
+                    b = torch.tensor(w.in_gpu_ids[i0:i0 + 256], device="cuda")
+                    ok = ok and bool(torch.equal(pool.view(torch.int16)[b], ref.view(torch.int16)[a]))
+            if overlapped:
+                for c in mig.calls:
+                    a = torch.tensor(c.ctx_idx, device="cuda")
+                    b = torch.tensor(c.dec_idx, device="cuda")
+                    ok = ok and bool(torch.equal(k_gpu.view(torch.int16)[b], src_k.view(torch.int16)[a]))
+                    ok = ok and bool(torch.equal(v_gpu.view(torch.int16)[b], src_v.view(torch.int16)[a]))
+            row = {"overlapped_with_migration": overlapped,
+                   "swap_out_GBps": round(bytes_dir / t_out / 1e9, 2),
+                   "swap_in_GBps": round(bytes_dir / t_in / 1e9, 2),
+                   "swap_out_frac_of_link": round(bytes_dir / t_out / 1e9 / link["d2h"], 4),
+                   "swap_in_frac_of_link": round(bytes_dir / t_in / 1e9 / link["h2d"], 4),
+                   "swap_out_ms": round(t_out * 1e3, 2), "swap_in_ms": round(t_in * 1e3, 2),
+                   "host_enqueue_swap_out_us": round(host_out_us, 1), "round_trip_bit_exact": ok}
+            if overlapped:
+                row["migration_ms_beside_swap_out"] = mig_ms[:3]
+                row["migration_ms_beside_swap_in"] = mig_ms[3:]
+                row["migration_ms_alone"] = round(migrate_alone_ms, 3)
+            rows.append(row)
+        results[mode_name] = rows
+    cabi.set_option("swap_mode", default_mode)
+    cabi.set_option("swap_wgs", default_wgs)
+    default_name = [n for n, m, g in variants if m == default_mode and (g is None or g == default_wgs)]
+    best = results[default_name[0] if default_name else variants[0][0]][1]
+    total_s = best["swap_out_ms"] * 1e-3 + best["swap_in_ms"] * 1e-3
+    cabi.reset()
+    return {
+        "metric": "KV swap GB/s (fraction of measured host link), LLaMA-2-7B shape, overlapped with an 8-request migration",
+        "value": round(2 * bytes_dir / total_s / 1e9, 2), "unit": "GB/s", "n_gpus": 1, "steps": 1, "warmup": 1,
+        "ms_per_step": round(total_s * 1e3, 2), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "u8", "data": "synthetic",
+        "config": {"workload": (f"{w.name}: {len(w.out_gpu_ids)} blocks x {2 * slab} B (K+V) out to a pinned pool of "
+                                f"{w.host_blocks} blocks and back into other slots of a {w.gpu_blocks}-block GPU pool; "
+                                f"concurrent migration of {len(mig.calls)} requests ({mig.total_blocks} blocks), seed {w.seed}"),
+                   "value_counts": "bytes over the host link, swap-out plus swap-in, default swap mode, overlapped run"},
+        "link_GBps": {k: round(v, 2) for k, v in link.items()},
+        "pin_host_pools_s": round(pin_s, 2),
+        "swap": results,
+        "roofline": {"bound": "host link", "achieved": round(2 * bytes_dir / total_s / 1e9, 2),
+                     "peak": round((link["d2h"] + link["h2d"]) / 2, 2), "unit": "GB/s",
+                     "frac": round(2 * bytes_dir / total_s / 1e9 / ((link["d2h"] + link["h2d"]) / 2), 4),
+                     "traffic": None},
+    }
 
 
 def verify(w, src_k, src_v, dst_k, dst_v) -> bool:

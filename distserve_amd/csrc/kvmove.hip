@@ -152,13 +152,12 @@ __device__ __forceinline__ void copy_rows(char *dst, const char *src, uint32_t n
     }
 }
 
-// grid = (tiles per block of one pool kind, blocks in this launch, 2 = {K, V}).
-// Everything up to the lane offset is wave-uniform: the segment, the block-index pair and
-// the tile's base addresses are scalar loads from the kernel-argument segment into SGPRs.
+// One tile of one block of one pool kind.  Everything up to the lane offset is
+// wave-uniform: the segment, the block-index pair and the tile's base addresses are scalar
+// loads from the kernel-argument segment into SGPRs.
 template <typename V, int THREADS, int UNROLL, bool NTL, bool NTS>
-__global__ __launch_bounds__(THREADS) void kvm_copy_kernel(const MigrateArgs a)
+__device__ __forceinline__ void do_tile(const MigrateArgs &a, uint32_t tile, uint32_t pair, bool is_v)
 {
-    uint32_t tile = blockIdx.x;
     uint32_t s = 0, tile_begin = 0;
     while (s + 1 < a.nseg && tile >= a.seg[s].tile_end) {
         tile_begin = a.seg[s].tile_end;
@@ -166,8 +165,7 @@ __global__ __launch_bounds__(THREADS) void kvm_copy_kernel(const MigrateArgs a)
     }
     tile -= tile_begin;
     const Seg &sg = a.seg[s];
-    const IdxPair ix = a.idx[blockIdx.y];
-    const bool is_v = blockIdx.z != 0;
+    const IdxPair ix = a.idx[pair];
 
     const char *src = (is_v ? sg.src_v : sg.src_k) + (uint64_t)(uint32_t)ix.ctx * sg.src_block_stride;
     char *dst = (is_v ? a.dst_v : a.dst_k) + (uint64_t)(uint32_t)ix.dec * a.dst_block_stride + sg.dst_off;
@@ -185,6 +183,28 @@ __global__ __launch_bounds__(THREADS) void kvm_copy_kernel(const MigrateArgs a)
         copy_rows<V, THREADS, UNROLL, NTL, NTS>(dst + (uint64_t)row0 * sg.dst_row_stride,
                                                 src + (uint64_t)row0 * sg.src_row_stride, nrows,
                                                 sg.run_bytes, sg.src_row_stride, sg.dst_row_stride);
+    }
+}
+
+// HBM-bound form: grid = (tiles per block of one pool kind, blocks in this launch, 2 = {K, V}),
+// one tile per workgroup, so that thousands of short-lived workgroups keep every channel busy.
+template <typename V, int THREADS, int UNROLL, bool NTL, bool NTS>
+__global__ __launch_bounds__(THREADS) void kvm_copy_kernel(const MigrateArgs a)
+{
+    do_tile<V, THREADS, UNROLL, NTL, NTS>(a, blockIdx.x, blockIdx.y, blockIdx.z != 0);
+}
+
+// Link-bound form: grid = (a few workgroups, 2 = {K, V}); each workgroup walks the
+// (block, tile) pairs of the launch with a stride of gridDim.x.  A copy that the host link
+// limits to tens of GB/s needs only a handful of workgroups in flight, and leaves the rest
+// of the GPU to whatever runs beside it.
+template <typename V>
+__global__ __launch_bounds__(256) void kvm_walk_kernel(const MigrateArgs a, uint32_t tiles_per_block)
+{
+    const uint32_t total = a.nidx * tiles_per_block;
+    for (uint32_t w = blockIdx.x; w < total; w += gridDim.x) {
+        const uint32_t pair = w / tiles_per_block;
+        do_tile<V, 256, 4, true, true>(a, w - pair * tiles_per_block, pair, blockIdx.y != 0);
     }
 }
 
@@ -217,7 +237,8 @@ std::atomic<int64_t> opt_threads{256};
 std::atomic<int64_t> opt_unroll{4};
 std::atomic<int64_t> opt_nt_load{1};
 std::atomic<int64_t> opt_nt_store{1};
-std::atomic<int64_t> opt_swap_mode{0};
+std::atomic<int64_t> opt_swap_mode{2};
+std::atomic<int64_t> opt_swap_wgs{4};
 
 std::atomic<int64_t> *find_opt(const char *name)
 {
@@ -228,6 +249,7 @@ std::atomic<int64_t> *find_opt(const char *name)
     if (!strcmp(name, "nt_load")) return &opt_nt_load;
     if (!strcmp(name, "nt_store")) return &opt_nt_store;
     if (!strcmp(name, "swap_mode")) return &opt_swap_mode;
+    if (!strcmp(name, "swap_wgs")) return &opt_swap_wgs;
     return nullptr;
 }
 
@@ -432,9 +454,21 @@ int build_plan(const KvmGeom *g, const void *dst_k, const void *dst_v, Plan *pla
 }
 
 // Enqueues the copy kernel over `segs` x `pairs`, as many launches as the 4 KiB argument needs.
+using WalkFn = void (*)(const MigrateArgs, uint32_t);
+
+WalkFn pick_walk(int vec)
+{
+    return vec == 16 ? kvm_walk_kernel<u32x4>
+         : vec == 8  ? kvm_walk_kernel<u32x2>
+         : vec == 4  ? kvm_walk_kernel<uint32_t>
+         : vec == 2  ? kvm_walk_kernel<uint16_t>
+                     : kvm_walk_kernel<uint8_t>;
+}
+
+// walk_wgs > 0 selects the link-bound form with that many workgroups per pool kind.
 int launch_copy(std::vector<Seg> segs, const IdxPair *pairs, int64_t n, char *dst_k, char *dst_v,
                 uint64_t dst_block_stride, int vec, hipStream_t stream, int64_t *out_launches,
-                int64_t *out_wgs_per_block, int *out_threads)
+                int64_t *out_wgs_per_block, int *out_threads, int walk_wgs = 0)
 {
     const Launch k = pick_kernel(vec);
     uint32_t tile_bytes = (uint32_t)opt_tile_bytes.load();
@@ -459,7 +493,13 @@ int launch_copy(std::vector<Seg> segs, const IdxPair *pairs, int64_t n, char *ds
             args.nidx = (uint32_t)std::min<int64_t>(kMaxIdx, n - i0);
             if (pairs) {
                 memcpy(args.idx, pairs + i0, args.nidx * sizeof(IdxPair));
-                hipLaunchKernelGGL(k.fn, dim3(tiles_total, args.nidx, 2), dim3(k.threads), 0, stream, args);
+                if (walk_wgs > 0) {
+                    const uint32_t work = tiles_total * args.nidx;
+                    hipLaunchKernelGGL(pick_walk(vec), dim3(std::min<uint32_t>((uint32_t)walk_wgs, work), 2),
+                                       dim3(256), 0, stream, args, tiles_total);
+                } else {
+                    hipLaunchKernelGGL(k.fn, dim3(tiles_total, args.nidx, 2), dim3(k.threads), 0, stream, args);
+                }
                 KVM_HIP(hipGetLastError());
             }
             ++launches;
@@ -558,6 +598,29 @@ int checked_pinned(const void *p, const char *what)
     return KVM_OK;
 }
 
+// A second stream (default priority) and the two events that fork it from and join it back
+// into the caller's stream; one set per device, made on first use, kept until the process ends.
+struct Fork {
+    hipStream_t side = nullptr;
+    hipEvent_t forked = nullptr, joined = nullptr;
+};
+std::mutex g_fork_mu;
+std::map<int, Fork> g_forks;
+
+int get_fork(Fork **out)
+{
+    int dev = 0;
+    KVM_HIP(hipGetDevice(&dev));
+    Fork &f = g_forks[dev];
+    if (!f.side) {
+        KVM_HIP(hipStreamCreateWithFlags(&f.side, hipStreamNonBlocking));
+        KVM_HIP(hipEventCreateWithFlags(&f.forked, hipEventDisableTiming));
+        KVM_HIP(hipEventCreateWithFlags(&f.joined, hipEventDisableTiming));
+    }
+    *out = &f;
+    return KVM_OK;
+}
+
 }  // namespace
 
 // ------------------------------------------------------------------------- C ABI
@@ -576,6 +639,8 @@ int kvm_set_option(const char *name, int64_t value)
     if (o == &opt_tile_bytes) ok = value >= 4096 && value <= (1 << 26) && (value & (value - 1)) == 0;
     else if (o == &opt_threads) ok = value == 256 || value == 512 || value == 1024;
     else if (o == &opt_unroll) ok = value == 1 || value == 2 || value == 4 || value == 8;
+    else if (o == &opt_swap_wgs) ok = value >= 1 && value <= 4096;
+    else if (o == &opt_swap_mode) ok = value >= 0 && value <= 2;
     else ok = value == 0 || value == 1;
     if (!ok) return fail(KVM_EINVAL, "value %lld is not valid for option '%s'", (long long)value, name);
     o->store(value);
@@ -755,11 +820,23 @@ int kvm_swap(const int64_t *src_ids, const int64_t *dst_ids, int64_t n, int is_s
         const int vec = vec_width((uint64_t)slab_bytes | (uintptr_t)src_k | (uintptr_t)src_v |
                                   (uintptr_t)dst_k | (uintptr_t)dst_v);
         return launch_copy({s}, pairs.data(), n, dst_k, dst_v, (uint64_t)slab_bytes, vec, st, nullptr,
-                           nullptr, nullptr);
+                           nullptr, nullptr, (int)opt_swap_wgs.load());
     }
 
-    // hipMemcpyAsync per run of blocks that are consecutive on both sides.
+    // hipMemcpyAsync per run of blocks that are consecutive on both sides.  In mode 2 the V
+    // pool's copies go to a second, library-owned stream forked from and joined back into
+    // the caller's stream, so that two copy engines work on one call.
     const hipMemcpyKind kind = is_swap_in ? hipMemcpyHostToDevice : hipMemcpyDeviceToHost;
+    hipStream_t st_v = st;
+    Fork *fork = nullptr;
+    std::unique_lock<std::mutex> fork_lock;
+    if (opt_swap_mode.load() == 2) {
+        fork_lock = std::unique_lock<std::mutex>(g_fork_mu);
+        if (int rc = get_fork(&fork)) return rc;
+        KVM_HIP(hipEventRecord(fork->forked, st));
+        KVM_HIP(hipStreamWaitEvent(fork->side, fork->forked, 0));
+        st_v = fork->side;
+    }
     int64_t i = 0;
     while (i < n) {
         int64_t j = i + 1;
@@ -768,8 +845,12 @@ int kvm_swap(const int64_t *src_ids, const int64_t *dst_ids, int64_t n, int is_s
         const size_t so = (size_t)pairs[i].ctx * (size_t)slab_bytes;
         const size_t dof = (size_t)pairs[i].dec * (size_t)slab_bytes;
         KVM_HIP(hipMemcpyAsync(dst_k + dof, src_k + so, bytes, kind, st));
-        KVM_HIP(hipMemcpyAsync(dst_v + dof, src_v + so, bytes, kind, st));
+        KVM_HIP(hipMemcpyAsync(dst_v + dof, src_v + so, bytes, kind, st_v));
         i = j;
+    }
+    if (fork) {
+        KVM_HIP(hipEventRecord(fork->joined, fork->side));
+        KVM_HIP(hipStreamWaitEvent(st, fork->joined, 0));
     }
     return KVM_OK;
 }

@@ -136,7 +136,12 @@ int kvm_copy_plain(void *dst, const void *src, int64_t nbytes, void *stream);
  *   "unroll"         16-byte vectors in flight per lane: 1, 2, 4 or 8
  *   "nt_load"        1 = nontemporal loads, 0 = plain
  *   "nt_store"       1 = nontemporal stores, 0 = plain
- *   "swap_mode"      0 = hipMemcpyAsync per contiguous run, 1 = copy kernel over pinned memory
+ *   "swap_mode"      2 (default) = hipMemcpyAsync per contiguous run, K pool on the caller's
+ *                    stream and V pool on a second stream forked from and joined back into it,
+ *                    0 = the same with both pools on the caller's stream,
+ *                    1 = copy kernel that reads/writes the pinned pools in place (fast alone,
+ *                        but it slows HBM-bound kernels that run beside it)
+ *   "swap_wgs"       workgroups per pool kind of the swap kernel (mode 1), 1..4096
  * kvm_get_option returns the value or KVM_EINVAL (as int64) for an unknown name.
  */
 int kvm_set_option(const char *name, int64_t value);
