@@ -19,7 +19,7 @@ for _path in (KVMOVE_LIB_PATH, TORCH_LIB_PATH):
     if not os.path.exists(_path):
         raise RuntimeError(
             f"Could not find {os.path.basename(_path)} at {_path}. "
-            "Build it first with `python -m distserve_amd.build` (hipcc, gfx950)."
+            "Build it first with `python distserve_amd/csrc/build.py` (hipcc, gfx950)."
         )
 
 torch.ops.load_library(TORCH_LIB_PATH)

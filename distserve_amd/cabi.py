@@ -24,7 +24,7 @@ KVM_HANDLE_WORDS = 8
 EXPORTS = (
     "kvm_version", "kvm_last_error", "kvm_get_mem_handle", "kvm_register_mem_handle",
     "kvm_register_source", "kvm_reset", "kvm_migrate", "kvm_swap", "kvm_copy_plain",
-    "kvm_set_option", "kvm_get_option", "kvm_migrate_plan",
+    "kvm_set_option", "kvm_get_option", "kvm_migrate_plan", "kvm_debug_divide",
 )
 
 
@@ -52,7 +52,7 @@ def _lib_path() -> str:
 def _load() -> ctypes.CDLL:
     path = _lib_path()
     if not os.path.exists(path):
-        raise RuntimeError(f"libkvmove.so not found at {path}; build it with `python -m distserve_amd.build`")
+        raise RuntimeError(f"libkvmove.so not found at {path}; build it with `python distserve_amd/csrc/build.py`")
     lib = ctypes.CDLL(path)
     i64, i32, vp, ip = ctypes.c_int64, ctypes.c_int32, ctypes.c_void_p, ctypes.POINTER(ctypes.c_int64)
     lib.kvm_version.restype = ctypes.c_int
@@ -68,9 +68,11 @@ def _load() -> ctypes.CDLL:
     lib.kvm_get_option.argtypes = [ctypes.c_char_p]
     lib.kvm_get_option.restype = i64
     lib.kvm_migrate_plan.argtypes = [ctypes.POINTER(KvmGeom), i64, vp, vp, ip]
+    lib.kvm_debug_divide.argtypes = [ctypes.c_uint32, ctypes.c_uint32]
+    lib.kvm_debug_divide.restype = ctypes.c_uint32
     for name in EXPORTS:
         fn = getattr(lib, name)
-        if name not in ("kvm_last_error", "kvm_get_option", "kvm_version"):
+        if name not in ("kvm_last_error", "kvm_get_option", "kvm_version", "kvm_debug_divide"):
             fn.restype = ctypes.c_int
     return lib
 

@@ -3,7 +3,9 @@
 ``libkvmove.so``        hand-written HIP kernels + the C ABI (``include/kvmove.h``); no torch.
 ``libkvmove_torch.so``  torch op shim registering ``block_migration_ops`` / ``swapping_ops``.
 
-Run as ``python -m distserve_amd.build``.  hipcc cross-compiles without a GPU.
+Run as ``python distserve_amd/csrc/build.py`` (a plain script on purpose: it must work
+when the libraries are missing or stale, so it does not import the package, which loads
+them).  hipcc cross-compiles without a GPU.
 """
 from __future__ import annotations
 
@@ -12,9 +14,9 @@ import shutil
 import subprocess
 import sys
 
-PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+CSRC_DIR = os.path.dirname(os.path.abspath(__file__))
+PKG_DIR = os.path.dirname(CSRC_DIR)
 REPO_DIR = os.path.dirname(PKG_DIR)
-CSRC_DIR = os.path.join(PKG_DIR, "csrc")
 LIB_DIR = os.path.join(PKG_DIR, "lib")
 INCLUDE_DIR = os.path.join(REPO_DIR, "include")
 

@@ -16,6 +16,7 @@
 #include <algorithm>
 #include <atomic>
 #include <cstdarg>
+#include <cstddef>
 #include <cstdio>
 #include <cstring>
 #include <map>
@@ -30,7 +31,7 @@ namespace {
 // ------------------------------------------------------------------ kernel argument
 
 constexpr int kMaxSegs = 8;    // source segments per launch
-constexpr int kMaxIdx = 440;   // block-index pairs per launch (keeps the argument <= 4 KiB)
+constexpr int kMaxIdx = 436;   // block-index pairs per launch (keeps the argument <= 4 KiB)
 
 // One rectangle of the decoding rank's block that a single context rank supplies:
 // n_rows runs of run_bytes, one per overlapping layer.
@@ -46,22 +47,26 @@ struct Seg {
     uint32_t rows_per_tile;    // >1 only when a whole row is smaller than a tile
     uint32_t pieces_per_row;   // >1 only when a row is larger than a tile
     uint32_t piece_bytes;
-    uint32_t tile_end;         // exclusive prefix sum of tiles over the launch's segments
-    uint32_t pad_;
+    uint32_t pieces_magic;     // tile / pieces_per_row without a divider: see fast_div
+    uint32_t pieces_shifts;
 };
-static_assert(sizeof(Seg) == 64, "Seg layout");
+static_assert(sizeof(Seg) == 64 && offsetof(Seg, src_row_stride) == 24 && offsetof(Seg, pieces_shifts) == 60,
+              "Seg layout: the kernel reads it as 16 dwords");
 
 struct IdxPair {
     int32_t ctx;  // block in the context pools
     int32_t dec;  // block in the decoding pool
 };
 
+// The first 64 bytes are everything a workgroup needs before it knows its segment; they
+// come in with one 16-dword scalar load.
 struct MigrateArgs {
     char *dst_k;
     char *dst_v;
     uint64_t dst_block_stride;
     uint32_t nseg;
     uint32_t nidx;
+    uint32_t tile_end[kMaxSegs];  // exclusive prefix sums of tiles per segment; UINT32_MAX past the last
     Seg seg[kMaxSegs];
     IdxPair idx[kMaxIdx];
 };
@@ -71,50 +76,76 @@ static_assert(sizeof(MigrateArgs) <= 4096, "kernel argument must stay within 4 K
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x16 __attribute__((ext_vector_type(16)));
 
-template <bool NT, typename V>
-__device__ __forceinline__ V ld(const V *p)
+__device__ __forceinline__ uint64_t u64_of(uint32_t lo, uint32_t hi) { return ((uint64_t)hi << 32) | lo; }
+
+// Kernel flavour bits (template parameter FLAGS).
+constexpr int kNtLoad = 1;      // nontemporal loads
+constexpr int kNtStore = 2;     // nontemporal stores
+constexpr int kWaveContig = 4;  // a wave's UNROLL vectors are adjacent in memory (else one pass apart)
+
+// Pool memory is addressed through global-address-space pointers, so that lanes issue
+// global_load/global_store (not flat ones) although the addresses are built from integers.
+#define KVM_GLOBAL __attribute__((address_space(1)))
+typedef KVM_GLOBAL char gchar;
+
+template <int FLAGS, typename V>
+__device__ __forceinline__ V ld(const KVM_GLOBAL V *p)
 {
-    if constexpr (NT) return __builtin_nontemporal_load(p);
+    if constexpr ((FLAGS & kNtLoad) != 0) return __builtin_nontemporal_load(p);
     else return *p;
 }
 
-template <bool NT, typename V>
-__device__ __forceinline__ void st(V *p, V v)
+template <int FLAGS, typename V>
+__device__ __forceinline__ void st(KVM_GLOBAL V *p, V v)
 {
-    if constexpr (NT) __builtin_nontemporal_store(v, p);
+    if constexpr ((FLAGS & kNtStore) != 0) __builtin_nontemporal_store(v, p);
     else *p = v;
 }
 
-// One contiguous run of `len` bytes (a multiple of sizeof(V)) by the whole workgroup:
-// UNROLL independent 16-byte loads per lane are issued before the first store.
-template <typename V, int THREADS, int UNROLL, bool NTL, bool NTS>
-__device__ __forceinline__ void copy_run(char *dst, const char *src, uint32_t len)
+// Byte offset, inside one step of THREADS*UNROLL vectors, of this lane's u-th vector.
+template <typename V, int THREADS, int UNROLL, int FLAGS>
+__device__ __forceinline__ uint32_t vec_off(int u)
 {
-    constexpr uint32_t kPass = THREADS * (uint32_t)sizeof(V);
-    constexpr uint32_t kStep = kPass * UNROLL;
-    const uint32_t lane_off = threadIdx.x * (uint32_t)sizeof(V);
+    constexpr uint32_t kVec = (uint32_t)sizeof(V);
+    if constexpr ((FLAGS & kWaveContig) != 0) {
+        const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+        return (wave * UNROLL + u) * (64 * kVec) + lane * kVec;
+    } else {
+        return (u * THREADS + threadIdx.x) * kVec;
+    }
+}
+
+// One contiguous run of `len` bytes (a multiple of sizeof(V)) by the whole workgroup:
+// UNROLL independent loads per lane are issued before the first store.  With
+// len <= THREADS * UNROLL * sizeof(V) the workgroup is "one shot": all loads, all stores,
+// end -- no wave ever waits for its own stores before it can load again.
+template <typename V, int THREADS, int UNROLL, int FLAGS>
+__device__ __forceinline__ void copy_run(gchar *dst, const gchar *src, uint32_t len)
+{
+    constexpr uint32_t kStep = THREADS * UNROLL * (uint32_t)sizeof(V);
     uint32_t off = 0;
     for (; off + kStep <= len; off += kStep) {
         V r[UNROLL];
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u)
-            r[u] = ld<NTL>(reinterpret_cast<const V *>(src + off + u * kPass + lane_off));
+            r[u] = ld<FLAGS>(reinterpret_cast<const KVM_GLOBAL V *>(src + off + vec_off<V, THREADS, UNROLL, FLAGS>(u)));
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u)
-            st<NTS>(reinterpret_cast<V *>(dst + off + u * kPass + lane_off), r[u]);
+            st<FLAGS>(reinterpret_cast<KVM_GLOBAL V *>(dst + off + vec_off<V, THREADS, UNROLL, FLAGS>(u)), r[u]);
     }
     if (off < len) {
         V r[UNROLL];
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
-            const uint32_t o = off + u * kPass + lane_off;
-            if (o < len) r[u] = ld<NTL>(reinterpret_cast<const V *>(src + o));
+            const uint32_t o = off + vec_off<V, THREADS, UNROLL, FLAGS>(u);
+            if (o < len) r[u] = ld<FLAGS>(reinterpret_cast<const KVM_GLOBAL V *>(src + o));
         }
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
-            const uint32_t o = off + u * kPass + lane_off;
-            if (o < len) st<NTS>(reinterpret_cast<V *>(dst + o), r[u]);
+            const uint32_t o = off + vec_off<V, THREADS, UNROLL, FLAGS>(u);
+            if (o < len) st<FLAGS>(reinterpret_cast<KVM_GLOBAL V *>(dst + o), r[u]);
         }
     }
 }
@@ -122,8 +153,8 @@ __device__ __forceinline__ void copy_run(char *dst, const char *src, uint32_t le
 // `nrows` runs of `len` bytes each, `sstride` / `dstride` apart: the UNROLL loads in
 // flight span row boundaries, so short rows still keep several loads outstanding.
 // The (row, pass-in-row) counters are wave-uniform and advance in SGPRs.
-template <typename V, int THREADS, int UNROLL, bool NTL, bool NTS>
-__device__ __forceinline__ void copy_rows(char *dst, const char *src, uint32_t nrows, uint32_t len,
+template <typename V, int THREADS, int UNROLL, int FLAGS>
+__device__ __forceinline__ void copy_rows(gchar *dst, const gchar *src, uint32_t nrows, uint32_t len,
                                           uint32_t sstride, uint32_t dstride)
 {
     constexpr uint32_t kPass = THREADS * (uint32_t)sizeof(V);
@@ -145,53 +176,75 @@ __device__ __forceinline__ void copy_rows(char *dst, const char *src, uint32_t n
         }
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u)
-            if (ok[u]) r[u] = ld<NTL>(reinterpret_cast<const V *>(src + soff[u]));
+            if (ok[u]) r[u] = ld<FLAGS>(reinterpret_cast<const KVM_GLOBAL V *>(src + soff[u]));
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u)
-            if (ok[u]) st<NTS>(reinterpret_cast<V *>(dst + doff[u]), r[u]);
+            if (ok[u]) st<FLAGS>(reinterpret_cast<KVM_GLOBAL V *>(dst + doff[u]), r[u]);
     }
 }
 
+// n / d for a divisor fixed on the host: magic and shifts from make_magic (round-up method
+// with a 33-bit multiplier folded into an add and two shifts; exact for every 32-bit n).
+__device__ __forceinline__ uint32_t fast_div(uint32_t n, uint32_t magic, uint32_t shifts)
+{
+    const uint32_t t = __umulhi(magic, n);
+    return (t + ((n - t) >> (shifts & 0xffu))) >> (shifts >> 8);
+}
+
 // One tile of one block of one pool kind.  Everything up to the lane offset is
-// wave-uniform: the segment, the block-index pair and the tile's base addresses are scalar
-// loads from the kernel-argument segment into SGPRs.
-template <typename V, int THREADS, int UNROLL, bool NTL, bool NTS>
+// wave-uniform and lives in SGPRs.  The scalar loads are arranged for a short dependent
+// chain, because a workgroup here lives for little more than one memory round trip: the
+// header (with every segment's tile range) and the block-index pair are independent
+// loads, the segment's fields are the one dependent round after them.
+template <typename V, int THREADS, int UNROLL, int FLAGS>
 __device__ __forceinline__ void do_tile(const MigrateArgs &a, uint32_t tile, uint32_t pair, bool is_v)
 {
+    // Two 64-byte records, each fetched whole with one 16-dword scalar load, so that the
+    // dependent chain is: {header, index pair} -> {segment} -> addresses.
+    static_assert(offsetof(MigrateArgs, tile_end) == 32 && offsetof(MigrateArgs, seg) == 64, "header layout");
+    const u32x16 h = *reinterpret_cast<const u32x16 *>(&a);
+    const IdxPair ix = a.idx[pair];
     uint32_t s = 0, tile_begin = 0;
-    while (s + 1 < a.nseg && tile >= a.seg[s].tile_end) {
-        tile_begin = a.seg[s].tile_end;
-        ++s;
+#pragma unroll
+    for (int j = 0; j < kMaxSegs - 1; ++j) {
+        if (tile >= h[8 + j]) {
+            s = j + 1;
+            tile_begin = h[8 + j];
+        }
     }
     tile -= tile_begin;
-    const Seg &sg = a.seg[s];
-    const IdxPair ix = a.idx[pair];
+    const u32x16 g = *reinterpret_cast<const u32x16 *>(&a.seg[s]);
+    const uint64_t src_base = is_v ? u64_of(g[2], g[3]) : u64_of(g[0], g[1]);
+    const uint64_t dst_base = is_v ? u64_of(h[2], h[3]) : u64_of(h[0], h[1]);
+    const uint64_t src_block_stride = u64_of(g[4], g[5]), dst_block_stride = u64_of(h[4], h[5]);
+    const uint32_t src_row_stride = g[6], dst_row_stride = g[7], dst_off = g[8], run_bytes = g[9];
+    const uint32_t n_rows = g[10], rows_per_tile = g[11], pieces_per_row = g[12], piece_bytes = g[13];
 
-    const char *src = (is_v ? sg.src_v : sg.src_k) + (uint64_t)(uint32_t)ix.ctx * sg.src_block_stride;
-    char *dst = (is_v ? a.dst_v : a.dst_k) + (uint64_t)(uint32_t)ix.dec * a.dst_block_stride + sg.dst_off;
+    const gchar *src = reinterpret_cast<const gchar *>(src_base + (uint64_t)(uint32_t)ix.ctx * src_block_stride);
+    gchar *dst = reinterpret_cast<gchar *>(dst_base + (uint64_t)(uint32_t)ix.dec * dst_block_stride + dst_off);
 
-    if (sg.rows_per_tile == 1) {
-        const uint32_t row = tile / sg.pieces_per_row;
-        const uint32_t piece = tile - row * sg.pieces_per_row;
-        const uint32_t col_off = piece * sg.piece_bytes;
-        const uint32_t len = min(sg.piece_bytes, sg.run_bytes - col_off);
-        copy_run<V, THREADS, UNROLL, NTL, NTS>(dst + (uint64_t)row * sg.dst_row_stride + col_off,
-                                               src + (uint64_t)row * sg.src_row_stride + col_off, len);
+    if (rows_per_tile == 1) {
+        const uint32_t row = fast_div(tile, g[14], g[15]);
+        const uint32_t piece = tile - row * pieces_per_row;
+        const uint32_t col_off = piece * piece_bytes;
+        const uint32_t len = min(piece_bytes, run_bytes - col_off);
+        copy_run<V, THREADS, UNROLL, FLAGS>(dst + (uint64_t)row * dst_row_stride + col_off,
+                                            src + (uint64_t)row * src_row_stride + col_off, len);
     } else {
-        const uint32_t row0 = tile * sg.rows_per_tile;
-        const uint32_t nrows = min(sg.rows_per_tile, sg.n_rows - row0);
-        copy_rows<V, THREADS, UNROLL, NTL, NTS>(dst + (uint64_t)row0 * sg.dst_row_stride,
-                                                src + (uint64_t)row0 * sg.src_row_stride, nrows,
-                                                sg.run_bytes, sg.src_row_stride, sg.dst_row_stride);
+        const uint32_t row0 = tile * rows_per_tile;
+        const uint32_t nrows = min(rows_per_tile, n_rows - row0);
+        copy_rows<V, THREADS, UNROLL, FLAGS>(dst + (uint64_t)row0 * dst_row_stride,
+                                             src + (uint64_t)row0 * src_row_stride, nrows, run_bytes,
+                                             src_row_stride, dst_row_stride);
     }
 }
 
 // HBM-bound form: grid = (tiles per block of one pool kind, blocks in this launch, 2 = {K, V}),
 // one tile per workgroup, so that thousands of short-lived workgroups keep every channel busy.
-template <typename V, int THREADS, int UNROLL, bool NTL, bool NTS>
+template <typename V, int THREADS, int UNROLL, int FLAGS>
 __global__ __launch_bounds__(THREADS) void kvm_copy_kernel(const MigrateArgs a)
 {
-    do_tile<V, THREADS, UNROLL, NTL, NTS>(a, blockIdx.x, blockIdx.y, blockIdx.z != 0);
+    do_tile<V, THREADS, UNROLL, FLAGS>(a, blockIdx.x, blockIdx.y, blockIdx.z != 0);
 }
 
 // Link-bound form: grid = (a few workgroups, 2 = {K, V}); each workgroup walks the
@@ -204,7 +257,7 @@ __global__ __launch_bounds__(256) void kvm_walk_kernel(const MigrateArgs a, uint
     const uint32_t total = a.nidx * tiles_per_block;
     for (uint32_t w = blockIdx.x; w < total; w += gridDim.x) {
         const uint32_t pair = w / tiles_per_block;
-        do_tile<V, 256, 4, true, true>(a, w - pair * tiles_per_block, pair, blockIdx.y != 0);
+        do_tile<V, 256, 4, kNtLoad | kNtStore>(a, w - pair * tiles_per_block, pair, blockIdx.y != 0);
     }
 }
 
@@ -232,13 +285,15 @@ int fail(int code, const char *fmt, ...)
 
 // ---- options
 
-std::atomic<int64_t> opt_tile_bytes{32768};
-std::atomic<int64_t> opt_threads{256};
-std::atomic<int64_t> opt_unroll{4};
+std::atomic<int64_t> opt_tile_bytes{0};
+std::atomic<int64_t> opt_threads{64};
+std::atomic<int64_t> opt_unroll{1};
 std::atomic<int64_t> opt_nt_load{1};
 std::atomic<int64_t> opt_nt_store{1};
 std::atomic<int64_t> opt_swap_mode{2};
 std::atomic<int64_t> opt_swap_wgs{4};
+std::atomic<int64_t> opt_lds_pad{0};
+std::atomic<int64_t> opt_wave_contig{0};
 
 std::atomic<int64_t> *find_opt(const char *name)
 {
@@ -250,6 +305,8 @@ std::atomic<int64_t> *find_opt(const char *name)
     if (!strcmp(name, "nt_store")) return &opt_nt_store;
     if (!strcmp(name, "swap_mode")) return &opt_swap_mode;
     if (!strcmp(name, "swap_wgs")) return &opt_swap_wgs;
+    if (!strcmp(name, "lds_pad")) return &opt_lds_pad;
+    if (!strcmp(name, "wave_contig")) return &opt_wave_contig;
     return nullptr;
 }
 
@@ -271,58 +328,68 @@ constexpr int64_t kHandleMagic = 0x4b564d4f56453031LL;  // "KVMOVE01"
 
 using KernelFn = void (*)(const MigrateArgs);
 
-template <typename V>
-KernelFn pick_narrow()
-{
-    return kvm_copy_kernel<V, 256, 4, true, true>;
-}
-
-template <int THREADS, int UNROLL>
-KernelFn pick_nt(bool ntl, bool nts)
-{
-    if (ntl) return nts ? kvm_copy_kernel<u32x4, THREADS, UNROLL, true, true>
-                        : kvm_copy_kernel<u32x4, THREADS, UNROLL, true, false>;
-    return nts ? kvm_copy_kernel<u32x4, THREADS, UNROLL, false, true>
-               : kvm_copy_kernel<u32x4, THREADS, UNROLL, false, false>;
-}
-
-template <int THREADS>
-KernelFn pick_unroll(int unroll, bool ntl, bool nts)
-{
-    switch (unroll) {
-    case 1: return pick_nt<THREADS, 1>(ntl, nts);
-    case 2: return pick_nt<THREADS, 2>(ntl, nts);
-    case 8: return pick_nt<THREADS, 8>(ntl, nts);
-    default: return pick_nt<THREADS, 4>(ntl, nts);
-    }
-}
-
-struct Launch {
+struct Variant {
+    int threads, unroll, flags;
     KernelFn fn;
-    int threads;
-    int vec;
 };
 
-Launch pick_kernel(int vec)
+#define KVM_VARIANT(T, U, F) {T, U, F, kvm_copy_kernel<u32x4, T, U, F>}
+#define KVM_VARIANT_ROW(T, F) \
+    KVM_VARIANT(T, 1, F), KVM_VARIANT(T, 2, F), KVM_VARIANT(T, 4, F), KVM_VARIANT(T, 8, F), KVM_VARIANT(T, 16, F)
+
+// 16-byte-vector flavours that are compiled in.  The exploration build (-DKVM_EXPLORE)
+// carries the whole grid for sweeps; the shipped library carries the one the sweeps chose
+// (64 lanes, one vector per lane: a single-wave workgroup that moves 1 KiB) plus a few
+// neighbours so that the tuning tests can show every flavour copies the same bytes.
+const Variant kVariants[] = {
+#ifdef KVM_EXPLORE
+    KVM_VARIANT_ROW(64, 3),   KVM_VARIANT_ROW(128, 3),  KVM_VARIANT_ROW(256, 3),
+    KVM_VARIANT_ROW(512, 3),  KVM_VARIANT_ROW(1024, 3),
+    KVM_VARIANT_ROW(64, 7),   KVM_VARIANT_ROW(128, 7),  KVM_VARIANT_ROW(256, 7),
+    KVM_VARIANT_ROW(512, 7),  KVM_VARIANT_ROW(1024, 7),
+    KVM_VARIANT(256, 4, 0),   KVM_VARIANT(256, 4, 1),   KVM_VARIANT(256, 4, 2),
+    KVM_VARIANT(256, 8, 0),   KVM_VARIANT(256, 8, 1),   KVM_VARIANT(256, 8, 2),
+#else
+    KVM_VARIANT(64, 1, 3),   KVM_VARIANT(64, 2, 3),   KVM_VARIANT(128, 1, 3),  KVM_VARIANT(256, 1, 3),
+    KVM_VARIANT(256, 4, 3),  KVM_VARIANT(256, 8, 3),  KVM_VARIANT(512, 2, 3),  KVM_VARIANT(512, 8, 3),
+    KVM_VARIANT(1024, 4, 3), KVM_VARIANT(64, 1, 0),   KVM_VARIANT(256, 4, 0),  KVM_VARIANT(512, 8, 0),
+    KVM_VARIANT(64, 4, 7),   KVM_VARIANT(256, 8, 7),
+#endif
+};
+
+struct Launch {
+    KernelFn fn = nullptr;
+    int threads = 0;
+    int unroll = 0;
+    int vec = 0;
+};
+
+int pick_kernel(int vec, Launch *l)
 {
-    Launch l;
-    l.vec = vec;
+    l->vec = vec;
     if (vec != 16) {
-        l.threads = 256;
-        l.fn = vec == 8 ? pick_narrow<u32x2>()
-             : vec == 4 ? pick_narrow<uint32_t>()
-             : vec == 2 ? pick_narrow<uint16_t>()
-                        : pick_narrow<uint8_t>();
-        return l;
+        // narrow vectors only serve odd shapes and misaligned pools: one flavour each
+        l->threads = 256;
+        l->unroll = 4;
+        l->fn = vec == 8 ? kvm_copy_kernel<u32x2, 256, 4, 3>
+              : vec == 4 ? kvm_copy_kernel<uint32_t, 256, 4, 3>
+              : vec == 2 ? kvm_copy_kernel<uint16_t, 256, 4, 3>
+                         : kvm_copy_kernel<uint8_t, 256, 4, 3>;
+        return KVM_OK;
     }
-    const int unroll = (int)opt_unroll.load();
-    const bool ntl = opt_nt_load.load() != 0, nts = opt_nt_store.load() != 0;
-    switch ((int)opt_threads.load()) {
-    case 512: l.threads = 512; l.fn = pick_unroll<512>(unroll, ntl, nts); break;
-    case 1024: l.threads = 1024; l.fn = pick_unroll<1024>(unroll, ntl, nts); break;
-    default: l.threads = 256; l.fn = pick_unroll<256>(unroll, ntl, nts); break;
+    const int threads = (int)opt_threads.load(), unroll = (int)opt_unroll.load();
+    const int flags = (opt_nt_load.load() ? kNtLoad : 0) | (opt_nt_store.load() ? kNtStore : 0) |
+                      (opt_wave_contig.load() ? kWaveContig : 0);
+    for (const Variant &v : kVariants) {
+        if (v.threads == threads && v.unroll == unroll && v.flags == flags) {
+            l->threads = threads;
+            l->unroll = unroll;
+            l->fn = v.fn;
+            return KVM_OK;
+        }
     }
-    return l;
+    return fail(KVM_EINVAL, "no kernel was built for threads=%d unroll=%d nt_load=%d nt_store=%d wave_contig=%d",
+                threads, unroll, flags & 1, (flags >> 1) & 1, (flags >> 2) & 1);
 }
 
 int vec_width(uint64_t bits)
@@ -331,6 +398,17 @@ int vec_width(uint64_t bits)
     for (int v = 16; v > 1; v >>= 1)
         if ((bits & (uint64_t)(v - 1)) == 0) return v;
     return 1;
+}
+
+// Multiplier and shifts with which fast_div divides by d (d >= 1).
+void make_magic(uint32_t d, uint32_t *magic, uint32_t *shifts)
+{
+    uint32_t l = 0;
+    while ((1ull << l) < d) ++l;                      // 2^(l-1) < d <= 2^l
+    const uint64_t m = ((1ull << 32) * ((1ull << l) - d)) / d + 1;
+    const uint32_t sh1 = l < 1 ? l : 1, sh2 = l - sh1;
+    *magic = (uint32_t)m;
+    *shifts = sh1 | (sh2 << 8);
 }
 
 // Splits a segment's rows into workgroup tiles of about tile_bytes.
@@ -348,6 +426,7 @@ void tile_segment(Seg &s, uint32_t tile_bytes, uint32_t *tiles)
         s.pieces_per_row = 1;
         *tiles = (s.n_rows + s.rows_per_tile - 1) / s.rows_per_tile;
     }
+    make_magic(s.pieces_per_row, &s.pieces_magic, &s.pieces_shifts);
 }
 
 // Folds rows that are back to back on both sides into one long run.
@@ -470,8 +549,11 @@ int launch_copy(std::vector<Seg> segs, const IdxPair *pairs, int64_t n, char *ds
                 uint64_t dst_block_stride, int vec, hipStream_t stream, int64_t *out_launches,
                 int64_t *out_wgs_per_block, int *out_threads, int walk_wgs = 0)
 {
-    const Launch k = pick_kernel(vec);
+    Launch k;
+    if (int rc = pick_kernel(vec, &k)) return rc;
+    // tile_bytes 0 = one shot: exactly what the workgroup's lanes hold in flight
     uint32_t tile_bytes = (uint32_t)opt_tile_bytes.load();
+    if (tile_bytes == 0) tile_bytes = (uint32_t)(k.threads * k.unroll * vec);
     int64_t launches = 0, wgs_per_block = 0;
     for (size_t s0 = 0; s0 < segs.size(); s0 += kMaxSegs) {
         MigrateArgs args;
@@ -485,9 +567,11 @@ int launch_copy(std::vector<Seg> segs, const IdxPair *pairs, int64_t n, char *ds
             uint32_t tiles = 0;
             tile_segment(s, tile_bytes, &tiles);
             tiles_total += tiles;
-            s.tile_end = tiles_total;
+            args.tile_end[j] = tiles_total;
             args.seg[j] = s;
         }
+        for (uint32_t j = args.nseg; j < kMaxSegs; ++j) args.tile_end[j] = UINT32_MAX;
+        args.tile_end[args.nseg - 1] = UINT32_MAX;   // nothing lies past the last segment
         wgs_per_block += 2 * (int64_t)tiles_total;
         for (int64_t i0 = 0; i0 < n; i0 += kMaxIdx) {
             args.nidx = (uint32_t)std::min<int64_t>(kMaxIdx, n - i0);
@@ -498,7 +582,8 @@ int launch_copy(std::vector<Seg> segs, const IdxPair *pairs, int64_t n, char *ds
                     hipLaunchKernelGGL(pick_walk(vec), dim3(std::min<uint32_t>((uint32_t)walk_wgs, work), 2),
                                        dim3(256), 0, stream, args, tiles_total);
                 } else {
-                    hipLaunchKernelGGL(k.fn, dim3(tiles_total, args.nidx, 2), dim3(k.threads), 0, stream, args);
+                    hipLaunchKernelGGL(k.fn, dim3(tiles_total, args.nidx, 2), dim3(k.threads),
+                                       (size_t)opt_lds_pad.load(), stream, args);
                 }
                 KVM_HIP(hipGetLastError());
             }
@@ -636,10 +721,11 @@ int kvm_set_option(const char *name, int64_t value)
     std::atomic<int64_t> *o = find_opt(name);
     if (!o) return fail(KVM_EINVAL, "unknown option '%s'", name ? name : "(null)");
     bool ok = true;
-    if (o == &opt_tile_bytes) ok = value >= 4096 && value <= (1 << 26) && (value & (value - 1)) == 0;
-    else if (o == &opt_threads) ok = value == 256 || value == 512 || value == 1024;
-    else if (o == &opt_unroll) ok = value == 1 || value == 2 || value == 4 || value == 8;
+    if (o == &opt_tile_bytes) ok = value == 0 || (value >= 1024 && value <= (1 << 26) && (value & (value - 1)) == 0);
+    else if (o == &opt_threads) ok = value == 64 || value == 128 || value == 256 || value == 512 || value == 1024;
+    else if (o == &opt_unroll) ok = value == 1 || value == 2 || value == 4 || value == 8 || value == 16;
     else if (o == &opt_swap_wgs) ok = value >= 1 && value <= 4096;
+    else if (o == &opt_lds_pad) ok = value >= 0 && value <= 65536;
     else if (o == &opt_swap_mode) ok = value >= 0 && value <= 2;
     else ok = value == 0 || value == 1;
     if (!ok) return fail(KVM_EINVAL, "value %lld is not valid for option '%s'", (long long)value, name);
@@ -853,6 +939,16 @@ int kvm_swap(const int64_t *src_ids, const int64_t *dst_ids, int64_t n, int is_s
         KVM_HIP(hipStreamWaitEvent(st, fork->joined, 0));
     }
     return KVM_OK;
+}
+
+uint32_t kvm_debug_divide(uint32_t n, uint32_t d)
+{
+    if (d == 0) return UINT32_MAX;
+    uint32_t magic = 0, shifts = 0;
+    make_magic(d, &magic, &shifts);
+    // the host twin of the device's fast_div
+    const uint32_t t = (uint32_t)(((uint64_t)magic * n) >> 32);
+    return (t + ((n - t) >> (shifts & 0xffu))) >> (shifts >> 8);
 }
 
 int kvm_copy_plain(void *dst, const void *src, int64_t nbytes, void *stream)

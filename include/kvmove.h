@@ -131,9 +131,15 @@ int kvm_copy_plain(void *dst, const void *src, int64_t nbytes, void *stream);
 
 /*
  * Tuning knobs (no counterpart in the reference).  Names:
- *   "tile_bytes"     payload bytes one workgroup moves per pool kind (power of two >= 4096)
- *   "threads"        workgroup size: 256, 512 or 1024
- *   "unroll"         16-byte vectors in flight per lane: 1, 2, 4 or 8
+ *   "tile_bytes"     payload bytes one workgroup moves per pool kind: 0 (default) = exactly
+ *                    what its lanes hold in flight, threads*unroll*16 ("one shot"), or a
+ *                    power of two >= 1024
+ *   "threads"        workgroup size: 64, 128, 256, 512 or 1024
+ *   "unroll"         16-byte vectors in flight per lane: 1, 2, 4, 8 or 16
+ *   "wave_contig"    1 = a wave's vectors are adjacent in memory, 0 = one pass apart
+ *   "lds_pad"        bytes of LDS requested per workgroup only to limit occupancy (0..65536)
+ *                    (not every threads/unroll/flag combination is compiled in; kvm_migrate
+ *                    reports KVM_EINVAL for one that is not)
  *   "nt_load"        1 = nontemporal loads, 0 = plain
  *   "nt_store"       1 = nontemporal stores, 0 = plain
  *   "swap_mode"      2 (default) = hipMemcpyAsync per contiguous run, K pool on the caller's
@@ -156,6 +162,13 @@ int64_t kvm_get_option(const char *name);
  */
 int kvm_migrate_plan(const KvmGeom *geom, int64_t n, const void *dst_k, const void *dst_v,
                      int64_t out[6]);
+
+/*
+ * Test hook (no counterpart in the reference): n / d computed the way the kernel computes
+ * a tile's row, with the multiplier and shifts the host derives for d.  Lets a CPU test
+ * check that arithmetic against plain division.  Returns UINT32_MAX for d == 0.
+ */
+uint32_t kvm_debug_divide(uint32_t n, uint32_t d);
 
 #ifdef __cplusplus
 }

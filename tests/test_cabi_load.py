@@ -25,12 +25,12 @@ def test_every_declared_symbol_is_exported(kvm):
 
 def test_version_and_options(kvm):
     assert kvm.version() >= 100
-    assert kvm.get_option("tile_bytes") >= 4096
+    assert kvm.get_option("tile_bytes") == 0 and kvm.get_option("threads") == 64 and kvm.get_option("unroll") == 1
     old = kvm.get_option("unroll")
     kvm.set_option("unroll", 8)
     assert kvm.get_option("unroll") == 8
     kvm.set_option("unroll", old)
-    for name, bad in (("tile_bytes", 5000), ("threads", 128), ("unroll", 3), ("nt_store", 2), ("nope", 1)):
+    for name, bad in (("tile_bytes", 5000), ("threads", 100), ("unroll", 3), ("nt_store", 2), ("nope", 1)):
         with pytest.raises(kvm.KvmError) as e:
             kvm.set_option(name, bad)
         assert e.value.code == kvm.KVM_EINVAL
@@ -79,3 +79,22 @@ def test_torch_ops_are_registered_with_the_reference_argument_order():
     z = torch.zeros(2, 1, 1, 2, 2, dtype=torch.float16)
     with pytest.raises(RuntimeError, match="GPU"):
         torch.ops.block_migration_ops.migrate_blocks(1, 1, [0], 1, 1, 0, 0, [0], z, z)
+
+
+def test_row_of_a_tile_is_computed_without_a_divider_exactly(kvm):
+    """The kernel finds a tile's row as tile / pieces_per_row with a host-made multiplier and
+    two shifts; the host twin of that arithmetic must equal plain division everywhere."""
+    import random
+
+    rng = random.Random(7)
+    divisors = list(range(1, 70)) + [80, 96, 127, 128, 129, 255, 256, 257, 1000, 4095, 4096, 4097, 65535, 65536,
+                                     65537, 2**20 - 1, 2**20, 2**20 + 1, 2**31 - 1, 2**31, 2**31 + 1, 2**32 - 1]
+    divisors += [rng.randrange(1, 2**32) for _ in range(200)]
+    for d in divisors:
+        probes = [0, 1, d - 1, d, d + 1, 2 * d - 1, 2 * d, 3 * d + 1, 2**31 - 1, 2**31, 2**32 - 1, 2**32 - d]
+        probes += [k * d + r for k in (5, 1023, 65535) for r in (0, d - 1)]
+        probes += [rng.randrange(0, 2**32) for _ in range(40)]
+        for n in probes:
+            if 0 <= n < 2**32:
+                assert kvm.lib.kvm_debug_divide(n, d) == n // d, (n, d)
+    assert kvm.lib.kvm_debug_divide(5, 0) == 2**32 - 1

@@ -96,9 +96,9 @@ def test_misaligned_pool_bases_pick_a_narrower_vector(kvm):
     kvm.reset()
 
 
-@pytest.mark.parametrize("n", [0, 1, 439, 440, 441, 881, 1000])
+@pytest.mark.parametrize("n", [0, 1, 435, 436, 437, 873, 1000])
 def test_list_lengths_around_the_per_launch_limit(kvm, n):
-    """One launch carries 440 index pairs; longer lists split into several launches."""
+    """One launch carries 436 index pairs; longer lists split into several launches."""
     g = oracle.Geom(2, 2, 16, 8, 2)
     gen = torch.Generator().manual_seed(n)
     ci = torch.randint(0, 64, (n,), generator=gen).tolist()          # context blocks may repeat
@@ -119,17 +119,23 @@ def test_more_context_ranks_than_one_launch_holds(kvm):
     kvm.reset()
 
 
-@pytest.mark.parametrize("tile_bytes,threads,unroll", [(4096, 256, 1), (8192, 512, 2), (32768, 256, 4),
-                                                       (65536, 1024, 8), (1 << 20, 512, 8), (16384, 1024, 4)])
-def test_every_tuning_choice_copies_the_same_bytes(kvm, tile_bytes, threads, unroll):
-    saved = {k: kvm.get_option(k) for k in ("tile_bytes", "threads", "unroll", "nt_load", "nt_store")}
+@pytest.mark.parametrize("tile_bytes,threads,unroll,flavours", [
+    (0, 64, 1, ((1, 1, 0), (0, 0, 0))),          # the default: one-shot single-wave workgroups
+    (0, 64, 2, ((1, 1, 0),)), (0, 128, 1, ((1, 1, 0),)), (4096, 256, 1, ((1, 1, 0),)),
+    (0, 256, 4, ((1, 1, 0), (0, 0, 0))), (32768, 256, 4, ((1, 1, 0),)), (0, 256, 8, ((1, 1, 0), (1, 1, 1))),
+    (8192, 512, 2, ((1, 1, 0),)), (1 << 20, 512, 8, ((1, 1, 0), (0, 0, 0))), (16384, 1024, 4, ((1, 1, 0),)),
+    (1024, 64, 4, ((1, 1, 1),)), (2048, 64, 1, ((1, 1, 0),))])
+def test_every_tuning_choice_copies_the_same_bytes(kvm, tile_bytes, threads, unroll, flavours):
+    names = ("tile_bytes", "threads", "unroll", "nt_load", "nt_store", "wave_contig")
+    saved = {k: kvm.get_option(k) for k in names}
     try:
         kvm.set_option("tile_bytes", tile_bytes)
         kvm.set_option("threads", threads)
         kvm.set_option("unroll", unroll)
-        for ntl, nts in ((1, 1), (0, 0)):
+        for ntl, nts, contig in flavours:
             kvm.set_option("nt_load", ntl)
             kvm.set_option("nt_store", nts)
+            kvm.set_option("wave_contig", contig)
             # 24 KiB rows (cfg1 shape), 80 KiB rows (TP2->1) and 8 KiB strided rows (GQA slice)
             check_case(kvm, oracle.Geom(3, 12, 16, 64, 2), 6, 7, [5, 1, 2], [0, 6, 3], seed=3)
             check_case(kvm, oracle.Geom(4, 40, 16, 128, 2, 1, 2, 1, 1), 4, 5, [3, 1], [0, 4], seed=4)
@@ -137,6 +143,25 @@ def test_every_tuning_choice_copies_the_same_bytes(kvm, tile_bytes, threads, unr
     finally:
         for k, v in saved.items():
             kvm.set_option(k, v)
+
+
+def test_a_flavour_that_was_not_built_is_refused(kvm):
+    g = oracle.Geom(2, 2, 16, 8, 2)
+    kvm.reset()
+    keep = upload_and_register(g, make_src_pools(g, 3, 1), make_src_pools(g, 3, 2))
+    dst = canary_pool(g.dec_pool_shape(3)).cuda()
+    old = kvm.get_option("unroll")
+    try:
+        kvm.set_option("unroll", 16)
+        with pytest.raises(kvm.KvmError) as e:
+            kvm.migrate(kvm_geom(g), [0], [1], dst.data_ptr(), dst.data_ptr(), 3, stream_handle())
+        assert e.value.code == kvm.KVM_EINVAL and "no kernel was built" in str(e.value)
+    finally:
+        kvm.set_option("unroll", old)
+    torch.cuda.synchronize()
+    assert same_bits(dst.cpu(), canary_pool(g.dec_pool_shape(3)))
+    del keep
+    kvm.reset()
 
 
 def test_errors_leave_the_destination_untouched(kvm):
