@@ -553,7 +553,7 @@ int launch_copy(std::vector<Seg> segs, const IdxPair *pairs, int64_t n, char *ds
     if (int rc = pick_kernel(vec, &k)) return rc;
     // tile_bytes 0 = one shot: exactly what the workgroup's lanes hold in flight
     uint32_t tile_bytes = (uint32_t)opt_tile_bytes.load();
-    if (tile_bytes == 0) tile_bytes = (uint32_t)(k.threads * k.unroll * vec);
+    if (tile_bytes == 0) tile_bytes = (uint32_t)((walk_wgs > 0 ? 256 * 4 : k.threads * k.unroll) * vec);
     int64_t launches = 0, wgs_per_block = 0;
     for (size_t s0 = 0; s0 < segs.size(); s0 += kMaxSegs) {
         MigrateArgs args;
