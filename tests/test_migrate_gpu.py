@@ -277,3 +277,138 @@ def test_config2_full_size_properties(kvm):
     assert same_bits(dst_k[torch.tensor(di, device="cuda")].cpu(), want_k)
     assert same_bits(dst_v[torch.tensor(di, device="cuda")].cpu(), want_v)
     kvm.reset()
+
+
+def test_migration_is_ordered_on_the_stream_it_is_given(kvm):
+    """Producer kernel -> migrate -> consumer kernel on one side stream, no host sync in
+    between: the copy must see the producer's data and the consumer must see the copy."""
+    g = oracle.Geom(4, 8, 16, 128, 2)
+    kvm.reset()
+    nb = 96
+    src_k = torch.zeros(g.ctx_pool_shape(nb), dtype=torch.float16, device="cuda")
+    src_v = torch.zeros_like(src_k)
+    fresh_k = make_src_pools(g, nb, 31)[0][0].cuda()
+    fresh_v = make_src_pools(g, nb, 32)[0][0].cuda()
+    dst_k = canary_pool(g.dec_pool_shape(nb)).cuda()
+    dst_v = canary_pool(g.dec_pool_shape(nb)).cuda()
+    kvm.register_source(1, 1, 0, 0, g.num_layers, g.num_kv_heads, src_k.data_ptr(), src_v.data_ptr(),
+                        src_k.numel() * 2)
+    gen = torch.Generator().manual_seed(3)
+    ci = torch.randperm(nb, generator=gen).tolist()
+    di = torch.randperm(nb, generator=gen).tolist()
+    side = torch.cuda.Stream()
+    torch.cuda.synchronize()
+    with torch.cuda.stream(side):
+        for _ in range(20):                       # keep the stream busy ahead of the producer
+            fresh_k.add_(0)
+        src_k.copy_(fresh_k)                      # producer: the "prefill" writes the blocks
+        src_v.copy_(fresh_v)
+        kvm.migrate(kvm_geom(g), ci, di, dst_k.data_ptr(), dst_v.data_ptr(), nb, side.cuda_stream)
+        seen_k, seen_v = dst_k.clone(), dst_v.clone()     # consumer
+    side.synchronize()
+    want_k, want_v = oracle_migrate(g, [[fresh_k.cpu()]], [[fresh_v.cpu()]], ci, di, nb)
+    assert same_bits(seen_k.cpu(), want_k) and same_bits(seen_v.cpu(), want_v)
+    kvm.reset()
+
+
+def test_calls_from_several_host_threads_on_their_own_streams(kvm):
+    """The library may be entered concurrently: four threads, each with its own stream and
+    its own destination pools, all reading the same registered source."""
+    import threading
+
+    g = oracle.Geom(2, 4, 16, 64, 2)
+    kvm.reset()
+    nb = 64
+    src_k, src_v = make_src_pools(g, nb, 41), make_src_pools(g, nb, 42)
+    keep = upload_and_register(g, src_k, src_v)
+    results, errors = {}, []
+
+    def work(tid):
+        try:
+            torch.cuda.set_device(0)
+            stream = torch.cuda.Stream()
+            gen = torch.Generator().manual_seed(100 + tid)
+            dk = canary_pool(g.dec_pool_shape(nb)).cuda()
+            dv = canary_pool(g.dec_pool_shape(nb)).cuda()
+            calls = []
+            for _ in range(25):
+                n = int(torch.randint(1, 9, (1,), generator=gen))
+                ci = torch.randint(0, nb, (n,), generator=gen).tolist()
+                di = torch.randperm(nb, generator=gen)[:n].tolist()
+                kvm.migrate(kvm_geom(g), ci, di, dk.data_ptr(), dv.data_ptr(), nb, stream.cuda_stream)
+                calls.append((ci, di))
+            stream.synchronize()
+            results[tid] = (dk.cpu(), dv.cpu(), calls)
+        except Exception as e:      # noqa: BLE001
+            errors.append((tid, repr(e)))
+
+    threads = [threading.Thread(target=work, args=(t,)) for t in range(4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    for tid, (dk, dv, calls) in results.items():
+        want_k, want_v = canary_pool(g.dec_pool_shape(nb)), canary_pool(g.dec_pool_shape(nb))
+        for ci, di in calls:
+            oracle.migrate_c(g, src_k, ci, di, want_k)
+            oracle.migrate_c(g, src_v, ci, di, want_v)
+        assert same_bits(dk, want_k) and same_bits(dv, want_v), tid
+    del keep
+    kvm.reset()
+
+
+@pytest.mark.parametrize("make", [workloads.config3, workloads.config4])
+def test_configs_3_and_4_full_size_properties(kvm, make):
+    """OPT-13B (TP2 -> TP1) and LLaMA-2-70B GQA (TP2/PP2 -> TP4 rank 1) at full size: after
+    every request's call, each of its blocks equals the source rectangles it was sliced from
+    (torch slicing + gather on the GPU); sampled blocks agree with the oracle on the CPU."""
+    w = make()
+    g = geom_of(w)
+    kvm.reset()
+    src_k = [[workloads.fill_uniform(w.src_pool_shape(), w.seed + 10 * p + t, "cuda") for t in range(w.ctx_tp)]
+             for p in range(w.ctx_pp)]
+    src_v = [[workloads.fill_uniform(w.src_pool_shape(), w.seed + 500 + 10 * p + t, "cuda") for t in range(w.ctx_tp)]
+             for p in range(w.ctx_pp)]
+    for p in range(w.ctx_pp):
+        for t in range(w.ctx_tp):
+            kvm.register_source(w.ctx_pp, w.ctx_tp, p, t, g.num_layers, g.num_kv_heads, src_k[p][t].data_ptr(),
+                                src_v[p][t].data_ptr(), src_k[p][t].numel() * 2)
+    dst_k = workloads.fill_canary(w.dst_pool_shape(), "cuda")
+    dst_v = workloads.fill_canary(w.dst_pool_shape(), "cuda")
+    l0, h0 = g.dec_pp_rank * g.dec_layers, g.dec_tp_rank * g.dec_heads
+    for n_call, call in enumerate(w.calls):
+        kvm.migrate(kvm_geom(g), call.ctx_idx, call.dec_idx, dst_k.data_ptr(), dst_v.data_ptr(), w.dst_blocks,
+                    stream_handle())
+        ctx = torch.tensor(call.ctx_idx, device="cuda")
+        dec = torch.tensor(call.dec_idx, device="cuda")
+        for src, dst in ((src_k, dst_k), (src_v, dst_v)):
+            got = dst.view(torch.int16)[dec]
+            for p in range(w.ctx_pp):
+                for t in range(w.ctx_tp):
+                    la, lb = max(l0, p * g.ctx_layers), min(l0 + g.dec_layers, (p + 1) * g.ctx_layers)
+                    ha, hb = max(h0, t * g.ctx_heads), min(h0 + g.dec_heads, (t + 1) * g.ctx_heads)
+                    if la >= lb or ha >= hb:
+                        continue
+                    want = src[p][t].view(torch.int16)[ctx, la - p * g.ctx_layers:lb - p * g.ctx_layers,
+                                                       ha - t * g.ctx_heads:hb - t * g.ctx_heads]
+                    assert torch.equal(got[:, la - l0:lb - l0, ha - h0:hb - h0], want), (call.request_id, p, t)
+        if n_call % 8 == 0:                                   # oracle on a sample of this call's blocks
+            pick = list(range(0, len(call.ctx_idx), max(1, len(call.ctx_idx) // 6)))[:6]
+            ci = [call.ctx_idx[i] for i in pick]
+            di = [call.dec_idx[i] for i in pick]
+            sel = torch.tensor(ci, device="cuda")
+            small_k = [[src_k[p][t][sel].cpu() for t in range(w.ctx_tp)] for p in range(w.ctx_pp)]
+            small_v = [[src_v[p][t][sel].cpu() for t in range(w.ctx_tp)] for p in range(w.ctx_pp)]
+            ident = list(range(len(pick)))
+            want_k, want_v = oracle_migrate(g, small_k, small_v, ident, ident, len(pick))
+            dsel = torch.tensor(di, device="cuda")
+            assert same_bits(dst_k[dsel].cpu(), want_k) and same_bits(dst_v[dsel].cpu(), want_v)
+    if not w.recycles_blocks:
+        touched = torch.zeros(w.dst_blocks, dtype=torch.bool, device="cuda")
+        touched[torch.tensor([b for c in w.calls for b in c.dec_idx], device="cuda")] = True
+        rest = (~touched).nonzero().flatten()
+        for dst in (dst_k, dst_v):
+            for i0 in range(0, rest.numel(), 128):
+                assert bool((dst.view(torch.int16)[rest[i0:i0 + 128]] == workloads.CANARY_BITS).all())
+    kvm.reset()
