@@ -35,7 +35,9 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--config", type=int, default=2, choices=[1, 2, 3, 4, 5])
-    ap.add_argument("--pattern", default="request", choices=["request", "batch"])
+    ap.add_argument("--pattern", default="request", choices=["request", "batch", "handoff", "handoff-batched"],
+                    help="handoff*: the same requests through Worker / BlockManager / the migration handoff "
+                         "(torch ops, block allocation and release included), one call per request or one per batch")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-verify", action="store_true")
     ap.add_argument("--opt", action="append", default=[], help="kvmove tuning option name=value")
@@ -165,6 +167,9 @@ def main():
         return
 
     w = {1: workloads.config1, 2: workloads.config2, 3: workloads.config3, 4: workloads.config4}[args.config]()
+    if args.pattern.startswith("handoff"):
+        print(json.dumps(run_handoff_bench(args, w)))
+        return
     torch.cuda.set_device(0)
     stream = torch.cuda.current_stream()
     s = w.shape
@@ -428,6 +433,93 @@ def run_swap_bench(args):
                      "peak": round((link["d2h"] + link["h2d"]) / 2, 2), "unit": "GB/s",
                      "frac": round(2 * bytes_dir / total_s / 1e9 / ((link["d2h"] + link["h2d"]) / 2), 4),
                      "traffic": None},
+    }
+
+
+def run_handoff_bench(args, w):
+    """The whole hand-off, not only the op: for every request allocate decoding blocks in the
+    BlockManager, call Worker.migrate_blocks (torch op -> C ABI -> kernel) on the decoding
+    worker, release the context blocks.  The free lists start in the workload's seeded order,
+    so the block tables are the same non-contiguous ones the default pattern uses.  Wall
+    clock from the first allocation to the GPU having finished the last copy."""
+    import torch
+
+    from distserve_amd import (CacheConfig, ContextStageLLMEngine, DecodingStageLLMEngine, ModelConfig,
+                               ParallelConfig, cabi, create_request, workloads)
+
+    assert not w.recycles_blocks and w.dec_pp == 1 and w.dec_tp == 1, "handoff patterns run configurations 1-3"
+    s = w.shape
+    model = ModelConfig.from_kv_shape(s.num_layers, s.num_kv_heads, s.head_dim, num_kv_heads=s.num_kv_heads)
+    cache = CacheConfig(s.block_size, 4096)
+    cabi.reset()
+    ctx = ContextStageLLMEngine(model, ParallelConfig(w.ctx_tp, 0, w.ctx_pp, 0), cache)
+    dec = DecodingStageLLMEngine(model, ParallelConfig(1, 0, 1, 0), cache,
+                                 clear_migrated_blocks_callback=ctx.clear_migrated_blocks_callback)
+    ctx._init_kvcache(w.src_blocks, 0)
+    dec._init_kvcache(w.dst_blocks, 0)
+    dec.register_kvcache_mem_handles(ctx.parallel_config, ctx.kv_cache_mem_handles)
+    for i, worker in enumerate(x for row in ctx.workers for x in row):
+        worker.k_cache.copy_(workloads.fill_uniform(worker.k_cache.shape, w.seed + i, "cuda"))
+        worker.v_cache.copy_(workloads.fill_uniform(worker.v_cache.shape, w.seed + 500 + i, "cuda"))
+    batched = args.pattern == "handoff-batched"
+
+    def seeded_free_lists():
+        used_src = [b for c in w.calls for b in c.ctx_idx]
+        used_dst = [b for c in w.calls for b in c.dec_idx]
+        ctx.block_manager.free_gpu_blocks_list[:] = used_src + sorted(set(range(w.src_blocks)) - set(used_src))
+        dec.block_manager.free_gpu_blocks_list[:] = used_dst + sorted(set(range(w.dst_blocks)) - set(used_dst))
+
+    def one_step(step):
+        seeded_free_lists()
+        migrating = []
+        for c in w.calls:
+            req = create_request(c.prompt_len, step * 1000 + c.request_id)
+            ctx.block_manager.allocate_blocks(req)
+            req.add_generated_token("t", 1)
+            migrating.append(ctx.on_prefill_finished(req))
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        if batched:
+            dec._migrate_blocks_batched(migrating)
+        else:
+            for m in migrating:
+                dec._migrate_blocks(m)
+        t1 = time.perf_counter()
+        torch.cuda.synchronize()
+        t2 = time.perf_counter()
+        tables = [(list(m.block_indexes), list(dec.block_manager.get_block_table(m.req.request_id))) for m in migrating]
+        for m in migrating:
+            dec.block_manager.free_blocks(m.req.request_id)
+        return t1 - t0, t2 - t0, tables
+
+    for i in range(args.warmup):
+        one_step(i)
+    host_s, total_s, tables = 0.0, 0.0, None
+    for i in range(args.steps):
+        h, t, tables = one_step(args.warmup + i)
+        host_s += h
+        total_s += t
+    # the tables the BlockManagers produced are the workload's own
+    same_tables = all(ci == c.ctx_idx and di == c.dec_idx for (ci, di), c in zip(tables, w.calls))
+    dw = dec.workers[0][0]
+    src_k = [[x.k_cache for x in row] for row in ctx.workers]
+    src_v = [[x.v_cache for x in row] for row in ctx.workers]
+    bit_exact = verify(w, src_k, src_v, dw.k_cache, dw.v_cache) if not args.no_verify else None
+    ms_per_step = total_s / args.steps * 1e3
+    hbm_gbps = 2 * w.payload_bytes / (ms_per_step * 1e-3) / 1e9
+    cabi.reset()
+    return {
+        "metric": f"KV migration hand-off GB/s + us/request, {w.name}", "value": round(hbm_gbps, 2), "unit": "GB/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u8", "data": "synthetic",
+        "config": {"workload": f"{w.name}: {len(w.calls)} requests, {w.total_blocks} blocks",
+                   "pattern": ("BlockManager.allocate_blocks + Worker.migrate_blocks (torch op) + release of the "
+                               "context blocks, " + ("one migrate call per batch" if batched else "one per request")),
+                   "value_counts": "HBM bytes read + written per second of host wall clock (allocation to GPU idle)"},
+        "us_per_request": round(ms_per_step * 1e3 / len(w.calls), 2),
+        "host_us_per_request": round(host_s / args.steps / len(w.calls) * 1e6, 2),
+        "frac_of_hbm_peak": round(hbm_gbps / HBM_PEAK_GBPS, 4),
+        "block_tables_equal_workload": same_tables, "bit_exact": bit_exact,
     }
 
 

@@ -101,10 +101,8 @@ class DecodingStageLLMEngine(SingleStageLLMEngine):
         self._remote_call_all_workers_async("register_kvcache_mem_handles", context_parallel_config,
                                             kv_cache_mem_handles)
 
-    def _migrate_blocks(self, migrating_req: MigratingRequest) -> None:
-        """Move one request from the context instance to this one (reference :490-536):
-        allocate blocks for its *prompt* here, have every decoding rank pull its share,
-        then release the blocks on the context side."""
+    def _allocate_for_migration(self, migrating_req: MigratingRequest) -> List[int]:
+        """Blocks on this side for the request's *prompt* (reference :505-517)."""
         req = migrating_req.req
         # the first generated token already exists; it must not count towards the blocks
         # that are allocated (and copied) now
@@ -114,18 +112,60 @@ class DecodingStageLLMEngine(SingleStageLLMEngine):
             self.block_manager.allocate_blocks(req)
         finally:
             req.generated_tokens, req.generated_token_ids = kept
-
         target_block_indexes = self.block_manager.get_block_table(req.request_id)
         assert len(target_block_indexes) == len(migrating_req.block_indexes), (
             f"request {req.request_id}: {len(migrating_req.block_indexes)} context blocks but "
             f"{len(target_block_indexes)} decoding blocks")
+        return target_block_indexes
 
+    def _release_source_blocks(self, migrating_reqs: List[MigratingRequest]) -> None:
+        if self.clear_migrated_blocks_callback is None:
+            return
+        events = [w.latest_migrate_event for row in self.workers for w in row
+                  if getattr(w, "latest_migrate_event", None) is not None]
+        for migrating_req in migrating_reqs:
+            self.clear_migrated_blocks_callback(migrating_req, events)
+
+    def _migrate_blocks(self, migrating_req: MigratingRequest) -> None:
+        """Move one request from the context instance to this one (reference :490-536):
+        allocate blocks for its *prompt* here, have every decoding rank pull its share,
+        then release the blocks on the context side."""
+        req = migrating_req.req
+        target_block_indexes = self._allocate_for_migration(migrating_req)
         self.lifetime_events.setdefault(req.request_id, []).append(("migration_begin", time.time()))
         self._remote_call_all_workers_async("migrate_blocks", migrating_req.block_indexes,
                                             migrating_req.context_parallel_config, target_block_indexes)
         self.lifetime_events[req.request_id].append(("migration_end", time.time()))
+        self._release_source_blocks([migrating_req])
 
-        if self.clear_migrated_blocks_callback is not None:
-            events = [w.latest_migrate_event for row in self.workers for w in row
-                      if getattr(w, "latest_migrate_event", None) is not None]
-            self.clear_migrated_blocks_callback(migrating_req, events)
+    def _migrate_blocks_batched(self, migrating_reqs: List[MigratingRequest], allocate_only: bool = False) -> None:
+        """Several requests of one context instance in ONE ``migrate_blocks`` call per worker:
+        their block tables are concatenated.  ``allocate_only`` does the allocation step for
+        requests whose copy is issued later together with others (the scheduler decides
+        acceptance request by request, each after the previous one's allocation)."""
+        if allocate_only:
+            for m in migrating_reqs:
+                self._allocate_for_migration(m)
+            return
+        if not migrating_reqs:
+            return
+        config = migrating_reqs[0].context_parallel_config
+        assert all(m.context_parallel_config.to_list()[0::2] == config.to_list()[0::2] for m in migrating_reqs), \
+            "requests migrated together must come from one context instance"
+        ctx_idx: List[int] = []
+        dec_idx: List[int] = []
+        now = time.time()
+        for m in migrating_reqs:
+            rid = m.req.request_id
+            if rid not in self.block_manager.block_table:
+                self._allocate_for_migration(m)
+            target = self.block_manager.get_block_table(rid)
+            assert len(target) == len(m.block_indexes)
+            ctx_idx += m.block_indexes
+            dec_idx += target
+            self.lifetime_events.setdefault(rid, []).append(("migration_begin", now))
+        self._remote_call_all_workers_async("migrate_blocks", ctx_idx, config, dec_idx)
+        now = time.time()
+        for m in migrating_reqs:
+            self.lifetime_events[m.req.request_id].append(("migration_end", now))
+        self._release_source_blocks(migrating_reqs)

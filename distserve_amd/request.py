@@ -43,6 +43,11 @@ class Request:
     def get_kvcache_slots(self) -> int:
         return self.get_input_len() + self.get_output_len()
 
+    def get_num_input_tokens(self) -> int:
+        """Tokens the next iteration feeds the model: the whole prompt in the context
+        stage, the last generated token afterwards (reference request.py:238-250)."""
+        return self.get_input_len() if self.is_context_stage() else 1
+
     def __repr__(self) -> str:
         return (f"Request(request_id={self.request_id}, input_len={self.get_input_len()}, "
                 f"output_len={self.get_output_len()})")
@@ -67,6 +72,15 @@ class BatchedRequests:
 
     def get_request_ids(self) -> List[int]:
         return [r.request_id for r in self.requests]
+
+    def get_num_input_tokens(self) -> int:
+        return sum(r.get_num_input_tokens() for r in self.requests)
+
+    def pop_finished_requests(self) -> List[Request]:
+        """Remove and return the finished requests (reference request.py:324-332)."""
+        finished = [r for r in self.requests if r.is_finished]
+        self.requests = [r for r in self.requests if not r.is_finished]
+        return finished
 
 
 class MigratingRequest:

@@ -112,3 +112,58 @@ def test_profile_and_block_bytes():
     assert worker._get_block_size_in_bytes(16, model, ParallelConfig(2, 0, 2, 0)) == 2 * 1024 * 1024
     n_gpu, n_cpu = worker._profile_num_available_blocks(16, 0.5, 2 << 30)
     assert n_cpu == 256 and n_gpu > 1000
+
+
+@pytest.mark.parametrize("batched", [False, True])
+def test_scheduler_driven_migration_matches_oracle(kvm, batched):
+    """Requests flow bridge queue -> scheduler.post_process -> engine -> op.  With
+    batch_migrations the accepted requests share ONE migrate call; the copied bytes and the
+    block tables are the same either way."""
+    from distserve_amd import DecodingStageFCFSScheduler, DecodingStageSchedConfig
+
+    kvm.reset()
+    model = ModelConfig.from_kv_shape(num_layers=4, num_heads=8, head_dim=64)
+    cache = CacheConfig(16, 64)
+    ctx = ContextStageLLMEngine(model, ParallelConfig(2, 0, 1, 0), cache)
+    dec = DecodingStageLLMEngine(model, ParallelConfig(1, 0, 1, 0), cache,
+                                 clear_migrated_blocks_callback=ctx.clear_migrated_blocks_callback)
+    ctx._init_kvcache(40, 0)
+    dec._init_kvcache(48, 8)
+    dec.register_kvcache_mem_handles(ctx.parallel_config, ctx.kv_cache_mem_handles)
+    for i, w in enumerate(ctx.workers[0]):
+        fill(w, 300 + 10 * i)
+    dw = dec.workers[0][0]
+    dw.k_cache.view(torch.int16).fill_(0x7C01)
+    dw.v_cache.view(torch.int16).fill_(0x7C01)
+    src_k = [[w.k_cache.cpu() for w in ctx.workers[0]]]
+    src_v = [[w.v_cache.cpu() for w in ctx.workers[0]]]
+    want_k, want_v = canary_pool(dw.k_cache.shape), canary_pool(dw.v_cache.shape)
+
+    calls = []
+    real = dw.migrate_blocks
+    dw.migrate_blocks = lambda ci, pc, di: (calls.append(len(ci)), real(ci, pc, di))[1]
+    sched = DecodingStageFCFSScheduler(
+        DecodingStageSchedConfig("fcfs", 8, 4096, waiting_block_prop_threshold=1.0), dec.parallel_config,
+        dec.block_manager, dec._migrate_blocks,
+        engine_migrate_blocks_batched_callback=dec._migrate_blocks_batched, batch_migrations=batched)
+    g = oracle.Geom(4, 8, 16, 64, 2, 1, 2, 1, 1)
+    tables = {}
+    for rid, prompt_len in enumerate([70, 16, 33, 120]):
+        req = create_request(prompt_len, rid)
+        ctx.block_manager.allocate_blocks(req)
+        req.add_generated_token("x", 1)
+        m = ctx.on_prefill_finished(req)
+        tables[rid] = list(m.block_indexes)
+        sched.add_request(m)
+    sched.post_process()
+    assert sched.unaccepted_queue == [] and [r.request_id for r in sched.waiting_queue] == [0, 1, 2, 3]
+    assert calls == ([5 + 1 + 3 + 8] if batched else [5, 1, 3, 8])
+    for rid, ci in tables.items():
+        di = dec.block_manager.get_block_table(rid)
+        oracle.migrate_c(g, src_k, ci, di, want_k)
+        oracle.migrate_c(g, src_v, ci, di, want_v)
+        assert rid not in ctx.block_manager.block_table
+    torch.cuda.synchronize()
+    assert same_bits(dw.k_cache.cpu(), want_k) and same_bits(dw.v_cache.cpu(), want_v)
+    assert [n for n, _ in dec.lifetime_events[3]] == ["migration_begin", "migration_end"]
+    kvm.reset()
