@@ -10,11 +10,11 @@ objects on one GPU and a "remote call" is a direct method call on every worker.
 """
 from __future__ import annotations
 
-import time
 from typing import Callable, Dict, List, Optional, Tuple
 
 from distserve_amd.block_manager import BlockManager
 from distserve_amd.config import CacheConfig, ModelConfig, ParallelConfig
+from distserve_amd.lifetime import LifetimeEvent, LifetimeEventType
 from distserve_amd.request import MigratingRequest, Request
 from distserve_amd.utils import MemoryHandle, Stage
 from distserve_amd.worker import Worker
@@ -89,10 +89,33 @@ class ContextStageLLMEngine(SingleStageLLMEngine):
 class DecodingStageLLMEngine(SingleStageLLMEngine):
     stage = Stage.DECODING
 
-    def __init__(self, *args, clear_migrated_blocks_callback: Optional[Callable] = None, **kwargs):
+    def __init__(self, *args, clear_migrated_blocks_callback: Optional[Callable] = None,
+                 engine_on_new_lifetime_event_callback: Optional[Callable] = None,
+                 gpu_complete_lifetime_events: bool = False, **kwargs):
         super().__init__(*args, **kwargs)
         self.clear_migrated_blocks_callback = clear_migrated_blocks_callback
-        self.lifetime_events: Dict[int, List[Tuple[str, float]]] = {}
+        self.engine_on_new_lifetime_event_callback = engine_on_new_lifetime_event_callback
+        # True: MigrationEnd is stamped after the copy's event has completed on the GPU
+        self.gpu_complete_lifetime_events = gpu_complete_lifetime_events
+        self.lifetime_events: Dict[int, List[LifetimeEvent]] = {}
+
+    def _lifetime(self, request_id: int, event_type: LifetimeEventType) -> None:
+        event = LifetimeEvent(event_type)
+        self.lifetime_events.setdefault(request_id, []).append(event)
+        if self.engine_on_new_lifetime_event_callback is not None:
+            self.engine_on_new_lifetime_event_callback(request_id, event)
+
+    def _wait_for_copies(self) -> None:
+        if not self.gpu_complete_lifetime_events:
+            return
+        for row in self.workers:
+            for w in row:
+                event = getattr(w, "latest_migrate_event", None)
+                if event is not None and hasattr(event, "synchronize"):
+                    event.synchronize()
+
+    def get_and_pop_request_lifetime_events(self, request_id: int) -> List[LifetimeEvent]:
+        return self.lifetime_events.pop(request_id, [])
 
     def register_kvcache_mem_handles(self, context_parallel_config: ParallelConfig,
                                      kv_cache_mem_handles: List[List[Tuple[MemoryHandle, MemoryHandle]]]) -> None:
@@ -132,10 +155,11 @@ class DecodingStageLLMEngine(SingleStageLLMEngine):
         then release the blocks on the context side."""
         req = migrating_req.req
         target_block_indexes = self._allocate_for_migration(migrating_req)
-        self.lifetime_events.setdefault(req.request_id, []).append(("migration_begin", time.time()))
+        self._lifetime(req.request_id, LifetimeEventType.MigrationBegin)
         self._remote_call_all_workers_async("migrate_blocks", migrating_req.block_indexes,
                                             migrating_req.context_parallel_config, target_block_indexes)
-        self.lifetime_events[req.request_id].append(("migration_end", time.time()))
+        self._wait_for_copies()
+        self._lifetime(req.request_id, LifetimeEventType.MigrationEnd)
         self._release_source_blocks([migrating_req])
 
     def _migrate_blocks_batched(self, migrating_reqs: List[MigratingRequest], allocate_only: bool = False) -> None:
@@ -154,7 +178,6 @@ class DecodingStageLLMEngine(SingleStageLLMEngine):
             "requests migrated together must come from one context instance"
         ctx_idx: List[int] = []
         dec_idx: List[int] = []
-        now = time.time()
         for m in migrating_reqs:
             rid = m.req.request_id
             if rid not in self.block_manager.block_table:
@@ -163,9 +186,9 @@ class DecodingStageLLMEngine(SingleStageLLMEngine):
             assert len(target) == len(m.block_indexes)
             ctx_idx += m.block_indexes
             dec_idx += target
-            self.lifetime_events.setdefault(rid, []).append(("migration_begin", now))
+            self._lifetime(rid, LifetimeEventType.MigrationBegin)
         self._remote_call_all_workers_async("migrate_blocks", ctx_idx, config, dec_idx)
-        now = time.time()
+        self._wait_for_copies()
         for m in migrating_reqs:
-            self.lifetime_events[m.req.request_id].append(("migration_end", now))
+            self._lifetime(m.req.request_id, LifetimeEventType.MigrationEnd)
         self._release_source_blocks(migrating_reqs)

@@ -90,7 +90,7 @@ def test_migrate_allocates_prompt_blocks_fans_out_then_frees_the_source(engines)
     assert len([k for k in kinds if k == "wait"]) == 4 * 4          # 4 events x 4 context workers
     assert 7 not in ctx.block_manager.block_table
     assert ctx.block_manager.free_gpu_blocks_list[-3:] == [1, 2, 3]
-    assert [n for n, _ in dec.lifetime_events[7]] == ["migration_begin", "migration_end"]
+    assert [str(e.event_type) for e in dec.lifetime_events[7]] == ["migration_begin", "migration_end"]
 
 
 def test_length_mismatch_is_refused_before_any_copy(engines):
@@ -103,3 +103,29 @@ def test_length_mismatch_is_refused_before_any_copy(engines):
     with pytest.raises(AssertionError):
         dec._migrate_blocks(m)
     assert not [e for e in LOG if e[0] == "migrate"]
+
+
+def test_lifetime_events_keep_the_reference_json_shape(engines):
+    from distserve_amd.lifetime import (LifetimeEvent, LifetimeEventType, json_decode_lifetime_events,
+                                        json_encode_lifetime_events, transmission_seconds)
+
+    ctx, dec = engines
+    seen = []
+    dec.engine_on_new_lifetime_event_callback = lambda rid, ev: seen.append((rid, str(ev.event_type)))
+    req = create_request(20, 11)
+    ctx.block_manager.allocate_blocks(req)
+    dec._migrate_blocks(ctx.on_prefill_finished(req))
+    assert seen == [(11, "migration_begin"), (11, "migration_end")]
+    events = dec.get_and_pop_request_lifetime_events(11)
+    assert 11 not in dec.lifetime_events
+    encoded = json_encode_lifetime_events(events)
+    assert [sorted(d) for d in encoded] == [["event_type", "timestamp"]] * 2
+    assert [d["event_type"] for d in encoded] == ["migration_begin", "migration_end"]
+    decoded = json_decode_lifetime_events(encoded)
+    assert [e.event_type for e in decoded] == [LifetimeEventType.MigrationBegin, LifetimeEventType.MigrationEnd]
+    assert transmission_seconds(decoded) == encoded[1]["timestamp"] - encoded[0]["timestamp"] >= 0
+    # every stage name of the reference is there
+    assert [str(t) for t in LifetimeEventType] == ["issued", "context_begin", "context_end", "migration_begin",
+                                                   "migration_end", "decoding_begin", "decoding_end"]
+    assert transmission_seconds([LifetimeEvent(LifetimeEventType.MigrationBegin, 1.0),
+                                 LifetimeEvent(LifetimeEventType.MigrationEnd, 1.5)]) == 0.5

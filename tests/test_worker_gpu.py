@@ -165,5 +165,55 @@ def test_scheduler_driven_migration_matches_oracle(kvm, batched):
         assert rid not in ctx.block_manager.block_table
     torch.cuda.synchronize()
     assert same_bits(dw.k_cache.cpu(), want_k) and same_bits(dw.v_cache.cpu(), want_v)
-    assert [n for n, _ in dec.lifetime_events[3]] == ["migration_begin", "migration_end"]
+    assert [str(e.event_type) for e in dec.lifetime_events[3]] == ["migration_begin", "migration_end"]
+    kvm.reset()
+
+
+def _paged_decode_attention(q, k_pool, v_pool, block_table, layer, n_tokens):
+    """What the forward pass does with the pools (reference worker.py:217-223 hands it
+    k_cache, v_cache and the block table): gather the request's blocks of one layer through
+    the block table, [block, head, slot, dim] -> [head, token, dim], attend."""
+    idx = torch.tensor(block_table, device=k_pool.device)
+    k = k_pool[idx, layer].permute(1, 0, 2, 3).reshape(k_pool.shape[2], -1, k_pool.shape[4])[:, :n_tokens].float()
+    v = v_pool[idx, layer].permute(1, 0, 2, 3).reshape(v_pool.shape[2], -1, v_pool.shape[4])[:, :n_tokens].float()
+    scores = torch.einsum("hd,htd->ht", q, k) / k.shape[-1] ** 0.5
+    return torch.einsum("ht,htd->hd", torch.softmax(scores, dim=-1), v)
+
+
+def test_consumer_reads_migrated_blocks_through_the_block_table(kvm):
+    """Consumer contract: paged attention over the decoding rank's pools + its block table
+    gives, head for head, what it gives over the context ranks' pools + their block table
+    (context TP2/PP2 -> decoding TP2: layers re-joined, heads re-split)."""
+    kvm.reset()
+    L, H, D, B = 4, 8, 64, 16
+    model = ModelConfig.from_kv_shape(L, H, D)
+    cache = CacheConfig(B, 64)
+    ctx = ContextStageLLMEngine(model, ParallelConfig(2, 0, 2, 0), cache)
+    dec = DecodingStageLLMEngine(model, ParallelConfig(2, 0, 1, 0), cache,
+                                 clear_migrated_blocks_callback=None)      # keep the source blocks
+    ctx._init_kvcache(20, 0)
+    dec._init_kvcache(24, 2)
+    dec.register_kvcache_mem_handles(ctx.parallel_config, ctx.kv_cache_mem_handles)
+    for i, w in enumerate(w for row in ctx.workers for w in row):
+        fill(w, 700 + 10 * i)
+    ctx.block_manager.allocate_blocks(create_request(40, 50))              # shift the tables apart
+    dec.block_manager.allocate_blocks(create_request(100, 51))
+    prompt_len = 75
+    req = create_request(prompt_len, 0)
+    ctx.block_manager.allocate_blocks(req)
+    m = ctx.on_prefill_finished(req)
+    ctx_table = list(m.block_indexes)
+    dec._migrate_blocks(m)
+    dec_table = dec.block_manager.get_block_table(0)
+    assert ctx_table != dec_table and len(dec_table) == 5
+    torch.cuda.synchronize()
+    q = (torch.rand((H, D), generator=torch.Generator().manual_seed(9)) * 2 - 1).cuda()
+    for layer in range(L):
+        p, ll = divmod(layer, L // 2)                                       # context pipeline rank, local layer
+        for u, dw in enumerate(dec.workers[0]):                             # decoding TP ranks: 4 heads each
+            heads = slice(u * 4, (u + 1) * 4)
+            got = _paged_decode_attention(q[heads], dw.k_cache, dw.v_cache, dec_table, layer, prompt_len)
+            cw = ctx.workers[p][u]                                          # context TP rank u owns the same heads
+            want = _paged_decode_attention(q[heads], cw.k_cache, cw.v_cache, ctx_table, ll, prompt_len)
+            assert torch.equal(got, want), (layer, u)
     kvm.reset()
