@@ -31,7 +31,7 @@ namespace {
 // ------------------------------------------------------------------ kernel argument
 
 constexpr int kMaxSegs = 8;    // source segments per launch
-constexpr int kMaxIdx = 436;   // block-index pairs per launch (keeps the argument <= 4 KiB)
+constexpr int kMaxIdx = 432;   // block-index pairs per launch (keeps the argument <= 4 KiB)
 
 // One rectangle of the decoding rank's block that a single context rank supplies:
 // n_rows runs of run_bytes, one per overlapping layer.
@@ -67,6 +67,13 @@ struct MigrateArgs {
     uint32_t nseg;
     uint32_t nidx;
     uint32_t tile_end[kMaxSegs];  // exclusive prefix sums of tiles per segment; UINT32_MAX past the last
+    // second header record: how a workgroup id becomes (block, tile)
+    uint32_t tiles_per_block;     // T: tiles of one block of one pool kind
+    uint32_t tiles_magic, tiles_shifts;
+    uint32_t chunk_tiles;         // C: consecutive work items one XCD takes at a time; 0 = ids in order
+    uint32_t chunk_magic, chunk_shifts;
+    uint32_t work;                // W = T * nidx work items per pool kind
+    uint32_t work_padded;         // grid.x / 2: W rounded up so that every XCD gets whole chunks
     Seg seg[kMaxSegs];
     IdxPair idx[kMaxIdx];
 };
@@ -76,6 +83,7 @@ static_assert(sizeof(MigrateArgs) <= 4096, "kernel argument must stay within 4 K
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x8 __attribute__((ext_vector_type(8)));
 typedef uint32_t u32x16 __attribute__((ext_vector_type(16)));
 
 __device__ __forceinline__ uint64_t u64_of(uint32_t lo, uint32_t hi) { return ((uint64_t)hi << 32) | lo; }
@@ -97,11 +105,24 @@ __device__ __forceinline__ V ld(const KVM_GLOBAL V *p)
     else return *p;
 }
 
+// Nontemporal stores of 16-byte vectors carry "sc1 nt" (streaming, written through beyond
+// the XCD's L2), which only inline assembly can express; beside nontemporal loads it
+// measured 0.5-2 % faster than "nt" alone.  Narrower vectors use the compiler's "nt".
+// The s_nop belongs to the store: a store of more than 8 bytes reads its data registers
+// for two more cycles, and the compiler, which cannot see that this text is such a store,
+// may otherwise reuse them at once.
 template <int FLAGS, typename V>
 __device__ __forceinline__ void st(KVM_GLOBAL V *p, V v)
 {
-    if constexpr ((FLAGS & kNtStore) != 0) __builtin_nontemporal_store(v, p);
-    else *p = v;
+    if constexpr ((FLAGS & kNtStore) != 0) {
+        if constexpr (sizeof(V) == 16) {
+            asm volatile("global_store_dwordx4 %0, %1, off sc1 nt\n\ts_nop 1" : : "v"(p), "v"(v) : "memory");
+        } else {
+            __builtin_nontemporal_store(v, p);
+        }
+    } else {
+        *p = v;
+    }
 }
 
 // Byte offset, inside one step of THREADS*UNROLL vectors, of this lane's u-th vector.
@@ -197,12 +218,13 @@ __device__ __forceinline__ uint32_t fast_div(uint32_t n, uint32_t magic, uint32_
 // header (with every segment's tile range) and the block-index pair are independent
 // loads, the segment's fields are the one dependent round after them.
 template <typename V, int THREADS, int UNROLL, int FLAGS>
-__device__ __forceinline__ void do_tile(const MigrateArgs &a, uint32_t tile, uint32_t pair, bool is_v)
+__device__ __forceinline__ void do_tile(const MigrateArgs &a, const u32x16 h, uint32_t tile, uint32_t pair, bool is_v)
 {
-    // Two 64-byte records, each fetched whole with one 16-dword scalar load, so that the
-    // dependent chain is: {header, index pair} -> {segment} -> addresses.
-    static_assert(offsetof(MigrateArgs, tile_end) == 32 && offsetof(MigrateArgs, seg) == 64, "header layout");
-    const u32x16 h = *reinterpret_cast<const u32x16 *>(&a);
+    // `h` is the first header record (64 bytes, one 16-dword scalar load by the caller); the
+    // segment is a second 64-byte record fetched whole, so that the dependent chain is
+    // {header records} -> {index pair, segment} -> addresses.
+    static_assert(offsetof(MigrateArgs, tile_end) == 32 && offsetof(MigrateArgs, tiles_per_block) == 64 &&
+                      offsetof(MigrateArgs, seg) == 96, "header layout");
     const IdxPair ix = a.idx[pair];
     uint32_t s = 0, tile_begin = 0;
 #pragma unroll
@@ -239,12 +261,75 @@ __device__ __forceinline__ void do_tile(const MigrateArgs &a, uint32_t tile, uin
     }
 }
 
-// HBM-bound form: grid = (tiles per block of one pool kind, blocks in this launch, 2 = {K, V}),
-// one tile per workgroup, so that thousands of short-lived workgroups keep every channel busy.
+// HBM-bound form: a 1-D grid of 2 * work_padded workgroups (K pool first, then V), one tile
+// per workgroup, so that thousands of short-lived workgroups keep every channel busy.
+//
+// Workgroup ids are dealt round-robin to the 8 XCDs.  With ids in order, every XCD would
+// touch every 8th KiB of every stream; instead id -> (xcd = id % 8, seq = id / 8) is turned
+// into a work item such that each XCD walks its own contiguous chunks of `chunk_tiles`
+// tiles (chunk number seq / C * 8 + xcd).  Chunks of 256 KiB and more measured 2-3 % faster
+// than in-order ids, chunks of 2-64 KiB 5-10 % slower.
 template <typename V, int THREADS, int UNROLL, int FLAGS>
 __global__ __launch_bounds__(THREADS) void kvm_copy_kernel(const MigrateArgs a)
 {
-    do_tile<V, THREADS, UNROLL, FLAGS>(a, blockIdx.x, blockIdx.y, blockIdx.z != 0);
+    // both header records in one round of scalar loads
+    const u32x16 h = *reinterpret_cast<const u32x16 *>(&a);
+    const u32x8 m = *reinterpret_cast<const u32x8 *>(&a.tiles_per_block);
+    const uint32_t tiles_per_block = m[0], chunk_tiles = m[3], work = m[6], work_padded = m[7];
+    uint32_t id = blockIdx.x;
+    const bool is_v = id >= work_padded;
+    if (is_v) id -= work_padded;
+    uint32_t w = id;
+    if (chunk_tiles != 0) {
+        const uint32_t xcd = id & 7u, seq = id >> 3;
+        const uint32_t q = fast_div(seq, m[4], m[5]);
+        w = (q * 8u + xcd) * chunk_tiles + (seq - q * chunk_tiles);
+    }
+    // Padding ids past the last chunk end here.  nidx (h[7]) is never 0; naming it in this
+    // test keeps the first record's load in the same round as the second's instead of
+    // behind the branch.
+    if (w >= work || h[7] == 0) return;
+    const uint32_t pair = fast_div(w, m[1], m[2]);
+    do_tile<V, THREADS, UNROLL, FLAGS>(a, h, w - pair * tiles_per_block, pair, is_v);
+}
+
+// The same for the plainest shape: one segment whose rows collapsed into a single run that
+// is a whole number of full tiles (context and decoding layouts agree, e.g. TP1 -> TP1).
+// Nothing depends on the tile's position but two multiplications, so the scalar prologue is
+// one round of loads for the three records, the index pair, and a dozen SALU instructions.
+template <typename V, int THREADS, int UNROLL, int FLAGS>
+__global__ __launch_bounds__(THREADS) void kvm_copy_simple_kernel(const MigrateArgs a)
+{
+    constexpr uint32_t kTile = THREADS * UNROLL * (uint32_t)sizeof(V);
+    const u32x16 h = *reinterpret_cast<const u32x16 *>(&a);
+    const u32x8 m = *reinterpret_cast<const u32x8 *>(&a.tiles_per_block);
+    const u32x16 g = *reinterpret_cast<const u32x16 *>(&a.seg[0]);
+    const uint32_t tiles_per_block = m[0], chunk_tiles = m[3], work = m[6], work_padded = m[7];
+    uint32_t id = blockIdx.x;
+    const bool is_v = id >= work_padded;
+    if (is_v) id -= work_padded;
+    uint32_t w = id;
+    if (chunk_tiles != 0) {
+        const uint32_t xcd = id & 7u, seq = id >> 3;
+        const uint32_t q = fast_div(seq, m[4], m[5]);
+        w = (q * 8u + xcd) * chunk_tiles + (seq - q * chunk_tiles);
+    }
+    if (w >= work || h[7] == 0 || g[10] == 0) return;   // (names h and g: see kvm_copy_kernel)
+    const uint32_t pair = fast_div(w, m[1], m[2]);
+    const uint32_t tile = w - pair * tiles_per_block;
+    const IdxPair ix = a.idx[pair];
+    const uint64_t src_base = is_v ? u64_of(g[2], g[3]) : u64_of(g[0], g[1]);
+    const uint64_t dst_base = is_v ? u64_of(h[2], h[3]) : u64_of(h[0], h[1]);
+    const uint64_t off = (uint64_t)tile * kTile;
+    const gchar *src = reinterpret_cast<const gchar *>(src_base + (uint64_t)(uint32_t)ix.ctx * u64_of(g[4], g[5]) + off);
+    gchar *dst = reinterpret_cast<gchar *>(dst_base + (uint64_t)(uint32_t)ix.dec * u64_of(h[4], h[5]) + g[8] + off);
+    V r[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u)
+        r[u] = ld<FLAGS>(reinterpret_cast<const KVM_GLOBAL V *>(src + vec_off<V, THREADS, UNROLL, FLAGS>(u)));
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u)
+        st<FLAGS>(reinterpret_cast<KVM_GLOBAL V *>(dst + vec_off<V, THREADS, UNROLL, FLAGS>(u)), r[u]);
 }
 
 // Link-bound form: grid = (a few workgroups, 2 = {K, V}); each workgroup walks the
@@ -257,7 +342,8 @@ __global__ __launch_bounds__(256) void kvm_walk_kernel(const MigrateArgs a, uint
     const uint32_t total = a.nidx * tiles_per_block;
     for (uint32_t w = blockIdx.x; w < total; w += gridDim.x) {
         const uint32_t pair = w / tiles_per_block;
-        do_tile<V, 256, 4, kNtLoad | kNtStore>(a, w - pair * tiles_per_block, pair, blockIdx.y != 0);
+        do_tile<V, 256, 4, kNtLoad | kNtStore>(a, *reinterpret_cast<const u32x16 *>(&a), w - pair * tiles_per_block,
+                                               pair, blockIdx.y != 0);
     }
 }
 
@@ -294,6 +380,8 @@ std::atomic<int64_t> opt_swap_mode{2};
 std::atomic<int64_t> opt_swap_wgs{4};
 std::atomic<int64_t> opt_lds_pad{0};
 std::atomic<int64_t> opt_wave_contig{0};
+std::atomic<int64_t> opt_xcd_map{1};
+std::atomic<int64_t> opt_simple{1};
 
 std::atomic<int64_t> *find_opt(const char *name)
 {
@@ -307,6 +395,8 @@ std::atomic<int64_t> *find_opt(const char *name)
     if (!strcmp(name, "swap_wgs")) return &opt_swap_wgs;
     if (!strcmp(name, "lds_pad")) return &opt_lds_pad;
     if (!strcmp(name, "wave_contig")) return &opt_wave_contig;
+    if (!strcmp(name, "xcd_map")) return &opt_xcd_map;
+    if (!strcmp(name, "simple")) return &opt_simple;
     return nullptr;
 }
 
@@ -330,10 +420,11 @@ using KernelFn = void (*)(const MigrateArgs);
 
 struct Variant {
     int threads, unroll, flags;
-    KernelFn fn;
+    KernelFn fn;         // any shape
+    KernelFn simple_fn;  // one collapsed segment of full tiles
 };
 
-#define KVM_VARIANT(T, U, F) {T, U, F, kvm_copy_kernel<u32x4, T, U, F>}
+#define KVM_VARIANT(T, U, F) {T, U, F, kvm_copy_kernel<u32x4, T, U, F>, kvm_copy_simple_kernel<u32x4, T, U, F>}
 #define KVM_VARIANT_ROW(T, F) \
     KVM_VARIANT(T, 1, F), KVM_VARIANT(T, 2, F), KVM_VARIANT(T, 4, F), KVM_VARIANT(T, 8, F), KVM_VARIANT(T, 16, F)
 
@@ -359,6 +450,7 @@ const Variant kVariants[] = {
 
 struct Launch {
     KernelFn fn = nullptr;
+    KernelFn simple_fn = nullptr;
     int threads = 0;
     int unroll = 0;
     int vec = 0;
@@ -385,6 +477,7 @@ int pick_kernel(int vec, Launch *l)
             l->threads = threads;
             l->unroll = unroll;
             l->fn = v.fn;
+            l->simple_fn = v.simple_fn;
             return KVM_OK;
         }
     }
@@ -533,6 +626,30 @@ int build_plan(const KvmGeom *g, const void *dst_k, const void *dst_v, Plan *pla
 }
 
 // Enqueues the copy kernel over `segs` x `pairs`, as many launches as the 4 KiB argument needs.
+// Fills the second header record: the id -> work item mapping for `tiles` tiles per block.
+void plan_work(MigrateArgs &args, uint32_t tiles, uint32_t tile_bytes)
+{
+    const uint32_t work = tiles * args.nidx;
+    args.tiles_per_block = tiles;
+    make_magic(tiles, &args.tiles_magic, &args.tiles_shifts);
+    args.work = work;
+    const int64_t mode = opt_xcd_map.load();
+    uint32_t chunk = 0;
+    if (mode != 0 && work >= 64) {
+        // an eighth of a block per XCD when that is at least 256 KiB, else an eighth of the launch
+        const bool block_eighth = tiles % 8 == 0 && (mode == 3 || (mode == 1 && (uint64_t)(tiles / 8) * tile_bytes >= (256u << 10)));
+        chunk = block_eighth ? tiles / 8 : (work + 7) / 8;
+    }
+    args.chunk_tiles = chunk;
+    if (chunk == 0) {
+        args.chunk_magic = args.chunk_shifts = 0;
+        args.work_padded = work;
+    } else {
+        make_magic(chunk, &args.chunk_magic, &args.chunk_shifts);
+        args.work_padded = (work + 8 * chunk - 1) / (8 * chunk) * (8 * chunk);
+    }
+}
+
 using WalkFn = void (*)(const MigrateArgs, uint32_t);
 
 WalkFn pick_walk(int vec)
@@ -573,8 +690,12 @@ int launch_copy(std::vector<Seg> segs, const IdxPair *pairs, int64_t n, char *ds
         for (uint32_t j = args.nseg; j < kMaxSegs; ++j) args.tile_end[j] = UINT32_MAX;
         args.tile_end[args.nseg - 1] = UINT32_MAX;   // nothing lies past the last segment
         wgs_per_block += 2 * (int64_t)tiles_total;
-        for (int64_t i0 = 0; i0 < n; i0 += kMaxIdx) {
-            args.nidx = (uint32_t)std::min<int64_t>(kMaxIdx, n - i0);
+        // a launch is a 1-D grid of 2 * tiles * blocks workgroups, which must stay below 2^31
+        if (tiles_total == 0 || tiles_total > (1u << 29))
+            return fail(KVM_EINVAL, "%u tiles per block cannot be launched", tiles_total);
+        const int64_t per_launch = std::min<int64_t>(kMaxIdx, (int64_t)((1u << 29) / tiles_total));
+        for (int64_t i0 = 0; i0 < n; i0 += per_launch) {
+            args.nidx = (uint32_t)std::min<int64_t>(per_launch, n - i0);
             if (pairs) {
                 memcpy(args.idx, pairs + i0, args.nidx * sizeof(IdxPair));
                 if (walk_wgs > 0) {
@@ -582,7 +703,12 @@ int launch_copy(std::vector<Seg> segs, const IdxPair *pairs, int64_t n, char *ds
                     hipLaunchKernelGGL(pick_walk(vec), dim3(std::min<uint32_t>((uint32_t)walk_wgs, work), 2),
                                        dim3(256), 0, stream, args, tiles_total);
                 } else {
-                    hipLaunchKernelGGL(k.fn, dim3(tiles_total, args.nidx, 2), dim3(k.threads),
+                    plan_work(args, tiles_total, tile_bytes);
+                    const Seg &s0 = args.seg[0];
+                    const bool simple = k.simple_fn && opt_simple.load() && args.nseg == 1 && s0.n_rows == 1 &&
+                                        s0.rows_per_tile == 1 && s0.run_bytes % tile_bytes == 0 &&
+                                        tile_bytes == (uint32_t)(k.threads * k.unroll * vec);
+                    hipLaunchKernelGGL(simple ? k.simple_fn : k.fn, dim3(2 * args.work_padded), dim3(k.threads),
                                        (size_t)opt_lds_pad.load(), stream, args);
                 }
                 KVM_HIP(hipGetLastError());
@@ -726,6 +852,7 @@ int kvm_set_option(const char *name, int64_t value)
     else if (o == &opt_unroll) ok = value == 1 || value == 2 || value == 4 || value == 8 || value == 16;
     else if (o == &opt_swap_wgs) ok = value >= 1 && value <= 4096;
     else if (o == &opt_lds_pad) ok = value >= 0 && value <= 65536;
+    else if (o == &opt_xcd_map) ok = value >= 0 && value <= 3;
     else if (o == &opt_swap_mode) ok = value >= 0 && value <= 2;
     else ok = value == 0 || value == 1;
     if (!ok) return fail(KVM_EINVAL, "value %lld is not valid for option '%s'", (long long)value, name);

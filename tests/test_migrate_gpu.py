@@ -96,9 +96,9 @@ def test_misaligned_pool_bases_pick_a_narrower_vector(kvm):
     kvm.reset()
 
 
-@pytest.mark.parametrize("n", [0, 1, 435, 436, 437, 873, 1000])
+@pytest.mark.parametrize("n", [0, 1, 431, 432, 433, 865, 1000])
 def test_list_lengths_around_the_per_launch_limit(kvm, n):
-    """One launch carries 436 index pairs; longer lists split into several launches."""
+    """One launch carries 432 index pairs; longer lists split into several launches."""
     g = oracle.Geom(2, 2, 16, 8, 2)
     gen = torch.Generator().manual_seed(n)
     ci = torch.randint(0, 64, (n,), generator=gen).tolist()          # context blocks may repeat
@@ -412,3 +412,26 @@ def test_configs_3_and_4_full_size_properties(kvm, make):
             for i0 in range(0, rest.numel(), 128):
                 assert bool((dst.view(torch.int16)[rest[i0:i0 + 128]] == workloads.CANARY_BITS).all())
     kvm.reset()
+
+
+@pytest.mark.parametrize("xcd_map,simple", [(0, 0), (0, 1), (1, 0), (1, 1), (2, 0), (2, 1), (3, 1)])
+def test_every_id_to_work_mapping_copies_the_same_bytes(kvm, xcd_map, simple):
+    """Workgroup ids are dealt to XCDs in contiguous chunks; with padding ids when the work
+    does not divide by 8 (odd tile counts, odd block counts)."""
+    saved = {k: kvm.get_option(k) for k in ("xcd_map", "simple")}
+    try:
+        kvm.set_option("xcd_map", xcd_map)
+        kvm.set_option("simple", simple)
+        gen = torch.Generator().manual_seed(17)
+        for g, nb_src, nb_dst, n in [
+                (oracle.Geom(2, 16, 16, 128, 2), 40, 48, 37),                   # 128 KiB blocks: 128 tiles
+                (oracle.Geom(1, 3, 16, 64, 2), 30, 31, 29),                     # 6 KiB blocks: 6 tiles, 29 blocks
+                (oracle.Geom(4, 40, 16, 128, 2, 1, 2, 1, 1), 12, 13, 11),       # two segments of 80 KiB rows
+                (oracle.Geom(12, 8, 16, 128, 2, 2, 2, 1, 4, 0, 1), 9, 10, 7),   # strided 8 KiB rows
+                (oracle.Geom(16, 32, 16, 128, 2), 6, 7, 5)]:                    # 2 MiB blocks: an eighth is 256 KiB
+            ci = torch.randint(0, nb_src, (n,), generator=gen).tolist()
+            di = torch.randperm(nb_dst, generator=gen)[:n].tolist()
+            check_case(kvm, g, nb_src, nb_dst, ci, di, seed=23)
+    finally:
+        for k, v in saved.items():
+            kvm.set_option(k, v)
