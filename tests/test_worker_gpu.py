@@ -217,3 +217,143 @@ def test_consumer_reads_migrated_blocks_through_the_block_table(kvm):
             want = _paged_decode_attention(q[heads], cw.k_cache, cw.v_cache, ctx_table, ll, prompt_len)
             assert torch.equal(got, want), (layer, u)
     kvm.reset()
+
+
+def test_random_serving_loop_against_an_oracle_mirror(kvm):
+    """A few hundred random steps of what the path sees in service -- prefill hand-offs
+    (TP2 -> TP1), swap-outs, swap-ins, frees -- through Worker, BlockManager and the hand-off,
+    mirrored step by step on CPU pools with the oracle; at the end every pool must agree
+    bit for bit."""
+    import random
+
+    kvm.reset()
+    rng = random.Random(1234)
+    L, H, D, B = 2, 8, 32, 16
+    model = ModelConfig.from_kv_shape(L, H, D)
+    cache = CacheConfig(B, 64)
+    ctx = ContextStageLLMEngine(model, ParallelConfig(2, 0, 1, 0), cache)
+    dec = DecodingStageLLMEngine(model, ParallelConfig(1, 0, 1, 0), cache,
+                                 clear_migrated_blocks_callback=ctx.clear_migrated_blocks_callback)
+    N_CTX, N_DEC, N_HOST = 48, 40, 32
+    ctx._init_kvcache(N_CTX, 0)
+    dec._init_kvcache(N_DEC, N_HOST)
+    dec.register_kvcache_mem_handles(ctx.parallel_config, ctx.kv_cache_mem_handles)
+    dw = dec.workers[0][0]
+    for t in (dw.k_cache, dw.v_cache):
+        t.view(torch.int16).fill_(0x7C01)
+    for t in (dw.k_swap, dw.v_swap):
+        t.view(torch.int16).fill_(0x7C01)
+    g = oracle.Geom(L, H, B, D, 2, 1, 2, 1, 1)
+    # the mirror
+    m_ctx_k = [[torch.zeros(w.k_cache.shape, dtype=torch.float16) for w in ctx.workers[0]]]
+    m_ctx_v = [[torch.zeros(w.v_cache.shape, dtype=torch.float16) for w in ctx.workers[0]]]
+    m_dec_k, m_dec_v = canary_pool(dw.k_cache.shape), canary_pool(dw.v_cache.shape)
+    m_host_k, m_host_v = canary_pool(dw.k_swap.shape), canary_pool(dw.v_swap.shape)
+    for t, w in enumerate(ctx.workers[0]):
+        w.k_cache.zero_()
+        w.v_cache.zero_()
+
+    live, next_id, seed = {}, 0, 1000
+    counts = {"migrate": 0, "swap_out": 0, "swap_in": 0, "free": 0}
+    for step in range(300):
+        on_gpu = [r for r in live.values() if dec.block_manager.get_location(r.request_id).value == "gpu"]
+        on_cpu = [r for r in live.values() if dec.block_manager.get_location(r.request_id).value == "cpu"]
+        op = rng.choice(["migrate", "migrate", "swap_out", "swap_in", "free"])
+        if op == "migrate":
+            prompt_len = rng.randint(1, 6 * B)
+            need = -(-prompt_len // B)
+            if need > ctx.block_manager.get_num_avail_gpu_blocks() or need > dec.block_manager.get_num_avail_gpu_blocks():
+                continue
+            req = create_request(prompt_len, next_id)
+            next_id += 1
+            ctx.block_manager.allocate_blocks(req)
+            table = ctx.block_manager.get_block_table(req.request_id)
+            # "prefill": fresh contents for the request's context blocks, on both sides
+            for t, w in enumerate(ctx.workers[0]):
+                seed += 1
+                fresh_k = rand_pool((len(table),) + tuple(w.k_cache.shape[1:]), seed)
+                fresh_v = rand_pool((len(table),) + tuple(w.v_cache.shape[1:]), seed + 50000)
+                idx = torch.tensor(table)
+                m_ctx_k[0][t][idx] = fresh_k
+                m_ctx_v[0][t][idx] = fresh_v
+                w.k_cache[idx.cuda()] = fresh_k.cuda()
+                w.v_cache[idx.cuda()] = fresh_v.cuda()
+            req.add_generated_token("t", 1)
+            mreq = ctx.on_prefill_finished(req)
+            ci = list(mreq.block_indexes)
+            dec._migrate_blocks(mreq)
+            di = list(dec.block_manager.get_block_table(req.request_id))
+            oracle.migrate_c(g, m_ctx_k, ci, di, m_dec_k)
+            oracle.migrate_c(g, m_ctx_v, ci, di, m_dec_v)
+            live[req.request_id] = req
+        elif op == "swap_out" and on_gpu:
+            req = rng.choice(on_gpu)
+            old = list(dec.block_manager.get_block_table(req.request_id))
+            if len(old) > dec.block_manager.get_num_avail_cpu_blocks():
+                continue
+            dec.block_manager.swap_out_requests([req])
+            new = list(dec.block_manager.get_block_table(req.request_id))
+            oracle.swap_c(old, new, m_dec_k, m_host_k)
+            oracle.swap_c(old, new, m_dec_v, m_host_v)
+        elif op == "swap_in" and on_cpu:
+            req = rng.choice(on_cpu)
+            old = list(dec.block_manager.get_block_table(req.request_id))
+            if len(old) > dec.block_manager.get_num_avail_gpu_blocks():
+                continue
+            dec.block_manager.swap_in_requests([req])
+            new = list(dec.block_manager.get_block_table(req.request_id))
+            oracle.swap_c(old, new, m_host_k, m_dec_k)
+            oracle.swap_c(old, new, m_host_v, m_dec_v)
+            dw.step([req.request_id])               # the compute stream waits for the swap-in
+        elif op == "free" and live:
+            req = rng.choice(list(live.values()))
+            dec._free_request_resources(req.request_id)
+            del live[req.request_id]
+        else:
+            continue
+        counts[op] += 1
+    torch.cuda.synchronize()
+    assert min(counts.values()) >= 10, counts
+    assert same_bits(dw.k_cache.cpu(), m_dec_k) and same_bits(dw.v_cache.cpu(), m_dec_v)
+    assert same_bits(dw.k_swap, m_host_k) and same_bits(dw.v_swap, m_host_v)
+    for t, w in enumerate(ctx.workers[0]):
+        assert same_bits(w.k_cache.cpu(), m_ctx_k[0][t]) and same_bits(w.v_cache.cpu(), m_ctx_v[0][t])
+    kvm.reset()
+
+
+def test_migrate_op_replays_inside_a_hip_graph(kvm):
+    """The op allocates nothing and only launches kernels on the current stream, so it can
+    be captured; every replay must copy what the sources hold at that time."""
+    kvm.reset()
+    g = oracle.Geom(2, 8, 16, 64, 2, 1, 2, 1, 1)
+    nb = 24
+    src_k = [[rand_pool(g.ctx_pool_shape(nb), 60 + t).cuda() for t in range(2)]]
+    src_v = [[rand_pool(g.ctx_pool_shape(nb), 70 + t).cuda() for t in range(2)]]
+    for t in range(2):
+        torch.ops.block_migration_ops.register_ipc_mem_handle(
+            torch.ops.block_migration_ops.get_ipc_mem_handle(src_k[0][t]),
+            torch.ops.block_migration_ops.get_ipc_mem_handle(src_v[0][t]), 2, 8, [2, t, 1, 0], [1, 0, 1, 0])
+    dst_k = canary_pool(g.dec_pool_shape(nb)).cuda()
+    dst_v = canary_pool(g.dec_pool_shape(nb)).cuda()
+    ci, di = [5, 0, 17, 9, 23], [1, 22, 4, 8, 0]
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):                   # warm-up outside the capture
+        torch.ops.block_migration_ops.migrate_blocks(1, 2, ci, 1, 1, 0, 0, di, dst_k, dst_v)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        torch.ops.block_migration_ops.migrate_blocks(1, 2, ci, 1, 1, 0, 0, di, dst_k, dst_v)
+    for replay in range(3):
+        for t in range(2):                          # new source contents, eager work between replays
+            src_k[0][t].copy_(rand_pool(g.ctx_pool_shape(nb), 100 * replay + t).cuda())
+            src_v[0][t].copy_(rand_pool(g.ctx_pool_shape(nb), 100 * replay + 10 + t).cuda())
+        dst_k.view(torch.int16).fill_(0x7C01)
+        dst_v.view(torch.int16).fill_(0x7C01)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        want_k, want_v = canary_pool(g.dec_pool_shape(nb)), canary_pool(g.dec_pool_shape(nb))
+        oracle.migrate_c(g, [[t.cpu() for t in src_k[0]]], ci, di, want_k)
+        oracle.migrate_c(g, [[t.cpu() for t in src_v[0]]], ci, di, want_v)
+        assert same_bits(dst_k.cpu(), want_k) and same_bits(dst_v.cpu(), want_v), replay
+    kvm.reset()
