@@ -413,6 +413,10 @@ def run_swap_bench(args):
         results[mode_name] = rows
     cabi.set_option("swap_mode", default_mode)
     cabi.set_option("swap_wgs", default_wgs)
+    cpu = None
+    if not args.no_cpu_baseline:
+        del k_ref, v_ref, src_k, src_v
+        cpu = swap_cpu_baseline(w)
     default_name = [n for n, m, g in variants if m == default_mode and (g is None or g == default_wgs)]
     best = results[default_name[0] if default_name else variants[0][0]][1]
     total_s = best["swap_out_ms"] * 1e-3 + best["swap_in_ms"] * 1e-3
@@ -429,11 +433,48 @@ def run_swap_bench(args):
         "link_GBps": {k: round(v, 2) for k, v in link.items()},
         "pin_host_pools_s": round(pin_s, 2),
         "swap": results,
+        "cpu_baseline": cpu,
         "roofline": {"bound": "host link", "achieved": round(2 * bytes_dir / total_s / 1e9, 2),
                      "peak": round((link["d2h"] + link["h2d"]) / 2, 2), "unit": "GB/s",
                      "frac": round(2 * bytes_dir / total_s / 1e9 / ((link["d2h"] + link["h2d"]) / 2), 4),
                      "traffic": None},
     }
+
+
+def swap_cpu_baseline(w, sample_blocks=256, budget_s=10.0):
+    """Reference semantics of the swap on the host: index_copy_(index_select) between two CPU
+    pools (oracle.swap_lib), out and back, on a sample of the block list with the pools
+    compacted to the sample (bytes per block unchanged)."""
+    import torch
+
+    import oracle
+    from distserve_amd import workloads
+
+    n = min(sample_blocks, len(w.out_gpu_ids))
+    gen = torch.Generator().manual_seed(w.seed)
+    a, b, c = (torch.randperm(n, generator=gen).tolist() for _ in range(3))
+    gpu_k = workloads.fill_uniform(w.shape.pool_shape(n), w.seed)
+    gpu_v = workloads.fill_uniform(w.shape.pool_shape(n), w.seed + 1)
+    host_k, host_v = workloads.fill_canary(w.shape.pool_shape(n)), workloads.fill_canary(w.shape.pool_shape(n))
+
+    def one_pass():
+        oracle.swap_lib(a, b, gpu_k, host_k)
+        oracle.swap_lib(a, b, gpu_v, host_v)
+        oracle.swap_lib(b, c, host_k, gpu_k)
+        oracle.swap_lib(b, c, host_v, gpu_v)
+
+    one_pass()
+    t0, passes = time.perf_counter(), 0
+    while time.perf_counter() - t0 < budget_s and passes < 50:
+        one_pass()
+        passes += 1
+    dt = time.perf_counter() - t0
+    moved = 2 * n * 2 * w.slab_bytes * passes            # out + in, K + V
+    return {"value": round(moved / dt / 1e9, 3), "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": (f"oracle.swap_lib (torch index_select/index_copy_ between CPU pools), {n} of "
+                       f"{len(w.out_gpu_ids)} blocks out and back, pools compacted to the sample, {passes} passes in "
+                       f"{dt:.1f} s; GB/s counts bytes copied, like the link figure"),
+            "host_cpu_count": os.cpu_count()}
 
 
 def run_handoff_bench(args, w):

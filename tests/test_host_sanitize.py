@@ -1,0 +1,29 @@
+"""Builds the C ABI's host code with AddressSanitizer and UBSan (host side only, the device
+code is compiled as usual) together with tests/host/abi_sanitize.cpp and runs it here: the
+argument-checking paths need no GPU."""
+import os
+import shutil
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.mark.skipif(shutil.which("hipcc") is None, reason="hipcc not on PATH")
+def test_abi_argument_paths_are_clean_under_asan_and_ubsan(tmp_path):
+    exe = tmp_path / "abi_sanitize"
+    cmd = ["hipcc", "--offload-arch=gfx950", "-O1", "-g", "-std=c++17",
+           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+           "-Xarch_host", "-fsanitize=address", "-Xarch_host", "-fsanitize=undefined",
+           "-Xarch_host", "-fno-sanitize-recover=undefined",
+           f"-I{os.path.join(ROOT, 'include')}",
+           os.path.join(ROOT, "distserve_amd", "csrc", "kvmove.hip"), "-x", "hip",
+           os.path.join(ROOT, "tests", "host", "abi_sanitize.cpp"), "-o", str(exe)]
+    build = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    assert build.returncode == 0, build.stdout[-3000:]
+    env = dict(os.environ, ASAN_OPTIONS="detect_leaks=0:abort_on_error=0", UBSAN_OPTIONS="print_stacktrace=1")
+    run = subprocess.run([str(exe)], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, env=env, timeout=300)
+    assert run.returncode == 0, run.stdout[-3000:]
+    assert "all checks passed" in run.stdout
+    assert "runtime error" not in run.stdout and "AddressSanitizer" not in run.stdout
