@@ -78,18 +78,21 @@ class Worker:
                 self.cache_config.block_size,
                 self.model_config.get_head_size())
 
+    def _new_pool(self, num_blocks: int, on_host: bool) -> torch.Tensor:
+        shape, dtype = self.kv_cache_shape(num_blocks), self.model_config.get_torch_dtype()
+        if on_host:
+            # pinned, so that the swap copies are asynchronous to the host
+            return torch.empty(shape, dtype=dtype, device="cpu", pin_memory=True)
+        return torch.empty(shape, dtype=dtype, device=self.device)
+
     def init_kvcache_and_swap(self, num_gpu_blocks: int, num_cpu_blocks: int) -> Tuple[MemoryHandle, MemoryHandle]:
-        """Allocate the K/V pools and the pinned swap pools; return the pools' memory handles
-        (reference worker.py:101-134)."""
-        dtype = self.model_config.get_torch_dtype()
-        self.k_cache = torch.empty(self.kv_cache_shape(num_gpu_blocks), dtype=dtype, device=self.device)
-        self.v_cache = torch.empty(self.kv_cache_shape(num_gpu_blocks), dtype=dtype, device=self.device)
-        # pinned, so that the swap copies are asynchronous to the host
-        self.k_swap = torch.empty(self.kv_cache_shape(num_cpu_blocks), dtype=dtype, device="cpu", pin_memory=True)
-        self.v_swap = torch.empty(self.kv_cache_shape(num_cpu_blocks), dtype=dtype, device="cpu", pin_memory=True)
+        """Allocate the K/V pools on HBM and the pinned K/V swap pools on the host; return the
+        memory handles of the two HBM pools (reference worker.py:101-134)."""
+        self.k_cache, self.v_cache = (self._new_pool(num_gpu_blocks, on_host=False) for _ in range(2))
+        self.k_swap, self.v_swap = (self._new_pool(num_cpu_blocks, on_host=True) for _ in range(2))
         torch.cuda.synchronize()
-        return (torch.ops.block_migration_ops.get_ipc_mem_handle(self.k_cache),
-                torch.ops.block_migration_ops.get_ipc_mem_handle(self.v_cache))
+        export = torch.ops.block_migration_ops.get_ipc_mem_handle
+        return export(self.k_cache), export(self.v_cache)
 
     def _get_block_size_in_bytes(self, block_size: int, model_config: ModelConfig,
                                  parallel_config: ParallelConfig) -> int:

@@ -357,3 +357,59 @@ def test_migrate_op_replays_inside_a_hip_graph(kvm):
         oracle.migrate_c(g, [[t.cpu() for t in src_v[0]]], ci, di, want_v)
         assert same_bits(dst_k.cpu(), want_k) and same_bits(dst_v.cpu(), want_v), replay
     kvm.reset()
+
+
+@pytest.mark.parametrize("dtype,block_size,head_dim", [("fp32", 16, 64), ("fp16", 8, 128), ("fp16", 32, 80),
+                                                       ("fp32", 4, 24)])
+def test_ops_with_other_dtypes_block_sizes_and_head_sizes(kvm, dtype, block_size, head_dim):
+    """fp32 pools (reference config.py:20-29 allows fp16 and fp32), block sizes other than 16
+    and head sizes that are not powers of two, through the torch ops and the Worker."""
+    kvm.reset()
+    model = ModelConfig.from_kv_shape(num_layers=4, num_heads=6, head_dim=head_dim, dtype=dtype)
+    cache = CacheConfig(block_size, 64)
+    ctx = ContextStageLLMEngine(model, ParallelConfig(3, 0, 2, 0), cache)          # TP3 / PP2
+    dec = DecodingStageLLMEngine(model, ParallelConfig(2, 0, 1, 0), cache,          # TP2
+                                 clear_migrated_blocks_callback=ctx.clear_migrated_blocks_callback)
+    ctx._init_kvcache(14, 0)
+    dec._init_kvcache(18, 6)
+    dec.register_kvcache_mem_handles(ctx.parallel_config, ctx.kv_cache_mem_handles)
+    tdtype = model.get_torch_dtype()
+    for i, w in enumerate(w for row in ctx.workers for w in row):
+        w.k_cache.copy_(rand_pool(w.k_cache.shape, 900 + i, tdtype))
+        w.v_cache.copy_(rand_pool(w.v_cache.shape, 950 + i, tdtype))
+    for w in dec.workers[0]:
+        oracle.bits(w.k_cache).fill_(0x7C01)
+        oracle.bits(w.v_cache).fill_(0x7C01)
+    src_k = [[w.k_cache.cpu() for w in row] for row in ctx.workers]
+    src_v = [[w.v_cache.cpu() for w in row] for row in ctx.workers]
+    want_k = [canary_pool(w.k_cache.shape, tdtype) for w in dec.workers[0]]
+    want_v = [canary_pool(w.v_cache.shape, tdtype) for w in dec.workers[0]]
+    ctx.block_manager.allocate_blocks(create_request(3 * block_size, 70))
+    for rid, prompt_len in enumerate([5 * block_size + 1, 1, 2 * block_size]):
+        req = create_request(prompt_len, rid)
+        ctx.block_manager.allocate_blocks(req)
+        m = ctx.on_prefill_finished(req)
+        ci = list(m.block_indexes)
+        dec._migrate_blocks(m)
+        di = dec.block_manager.get_block_table(rid)
+        for u in range(2):
+            g = oracle.Geom(4, 6, block_size, head_dim, model.get_dtype_size(), 2, 3, 1, 2, 0, u)
+            oracle.migrate_c(g, src_k, ci, di, want_k[u])
+            oracle.migrate_c(g, src_v, ci, di, want_v[u])
+    # and a swap round trip of request 0 on both decoding ranks
+    req0 = create_request(5 * block_size + 1, 0)
+    old = list(dec.block_manager.get_block_table(0))
+    dec.block_manager.swap_out_requests([req0])
+    host = list(dec.block_manager.get_block_table(0))
+    dec.block_manager.swap_in_requests([req0])
+    new = list(dec.block_manager.get_block_table(0))
+    for u, w in enumerate(dec.workers[0]):
+        hk, hv = canary_pool(w.k_swap.shape, tdtype), canary_pool(w.v_swap.shape, tdtype)
+        oracle.swap_c(old, host, want_k[u], hk)
+        oracle.swap_c(old, host, want_v[u], hv)
+        oracle.swap_c(host, new, hk, want_k[u])
+        oracle.swap_c(host, new, hv, want_v[u])
+    torch.cuda.synchronize()
+    for u, w in enumerate(dec.workers[0]):
+        assert same_bits(w.k_cache.cpu(), want_k[u]) and same_bits(w.v_cache.cpu(), want_v[u]), u
+    kvm.reset()
