@@ -1,11 +1,13 @@
 // kvmove.hip -- KV-block migration and swap for MI355X (gfx950, wave64).
 //
-// The whole path is byte movement, so there is no MFMA here.  One copy kernel serves
-// migration (gather by block-index tables + re-slice of layers/heads between the context
-// instance's TP/PP layout and one decoding rank), the kernel flavour of swap, and the
-// plain calibration copy.  Its metadata (segment table and block-index pairs) travels in
-// the kernel-argument segment, so every workgroup picks it up with scalar loads into
-// SGPRs and no device-side table, staging copy or allocation exists anywhere on the path.
+// The whole path is byte movement, so there is no MFMA here.  One piece of tile-copy code
+// serves migration (gather by block-index tables + re-slice of layers/heads between the
+// context instance's TP/PP layout and one decoding rank), the kernel flavour of swap, and
+// the plain calibration copy, in three launch forms: kvm_copy_kernel (any shape),
+// kvm_copy_simple_kernel (layouts that agree) and kvm_walk_kernel (link-bound).  The
+// metadata (segment table and block-index pairs) travels in the kernel-argument segment,
+// so every workgroup picks it up with scalar loads into SGPRs and no device-side table,
+// staging copy or allocation exists anywhere on the path.
 //
 // Reference call sites this stands behind: distserve/worker.py:133-134 (handles),
 // :239-246 (registration), :250-267 (migrate_blocks), :303-311 (swap).
@@ -1083,7 +1085,7 @@ int kvm_copy_plain(void *dst, const void *src, int64_t nbytes, void *stream)
     if (!dst || !src || nbytes < 0) return fail(KVM_EINVAL, "kvm_copy_plain: null pointer or negative size");
     if (nbytes == 0) return KVM_OK;
     // Expressed as one segment over 4 MiB "blocks" with identity index pairs; K and V
-    // stand for the two halves of the buffer so that both grid planes do work.
+    // stand for the two halves of the buffer, as they stand for the two pools elsewhere.
     const int64_t chunk = 4ll << 20;
     const int64_t half_chunks = nbytes / (2 * chunk);
     const int vec = vec_width((uint64_t)(uintptr_t)dst | (uint64_t)(uintptr_t)src | (uint64_t)nbytes);
