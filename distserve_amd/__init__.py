@@ -30,6 +30,8 @@ from distserve_amd.config import CacheConfig, DisaggParallelConfig, ModelConfig,
 from distserve_amd.request import MigratingRequest, Request, create_request  # noqa: E402
 from distserve_amd.worker import ParaWorker, Worker  # noqa: E402
 from distserve_amd.handoff import ContextStageLLMEngine, DecodingStageLLMEngine  # noqa: E402
+from distserve_amd.context_stage_scheduler import (  # noqa: E402
+    ContextStageFCFSScheduler, ContextStageSchedConfig, get_context_stage_scheduler)
 from distserve_amd.decoding_stage_scheduler import (  # noqa: E402
     DecodingStageFCFSScheduler, DecodingStageSchedConfig, get_decoding_stage_scheduler)
 
@@ -37,5 +39,6 @@ __all__ = [
     "cabi", "BlockLocation", "BlockManager", "CacheConfig", "DisaggParallelConfig", "ModelConfig",
     "ParallelConfig", "MigratingRequest", "Request", "create_request", "ParaWorker", "Worker",
     "ContextStageLLMEngine", "DecodingStageLLMEngine", "DecodingStageFCFSScheduler",
-    "DecodingStageSchedConfig", "get_decoding_stage_scheduler",
+    "DecodingStageSchedConfig", "get_decoding_stage_scheduler", "ContextStageFCFSScheduler",
+    "ContextStageSchedConfig", "get_context_stage_scheduler",
 ]

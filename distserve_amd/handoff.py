@@ -69,6 +69,7 @@ class ContextStageLLMEngine(SingleStageLLMEngine):
     def __init__(self, *args, **kwargs):
         super().__init__(*args, **kwargs)
         self.bridge_queue: List[MigratingRequest] = []
+        self.scheduler = None     # optional ContextStageFCFSScheduler, told when a request has left
 
     def on_prefill_finished(self, request: Request) -> MigratingRequest:
         """Tail of the context step: the request's blocks stay where they are and their
@@ -84,6 +85,8 @@ class ContextStageLLMEngine(SingleStageLLMEngine):
         for event in migrate_events:
             self._remote_call_all_workers_async("wait_stream_for_migration", event)
         self._free_request_resources(migrated_request.req.request_id)
+        if self.scheduler is not None:
+            self.scheduler.on_request_migrated(migrated_request)
 
 
 class DecodingStageLLMEngine(SingleStageLLMEngine):
