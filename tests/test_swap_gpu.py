@@ -141,3 +141,61 @@ def test_config5_shape_swap_overlapping_a_migration(kvm, swap_mode):
         assert a != b and same_bits(k_gpu[b].cpu(), k0[a])
     del keep
     kvm.reset()
+
+
+def test_config5_full_size_round_trip_beside_a_migration(kvm):
+    """Configuration 5 at full size with the default swap mode: 2048 blocks of the
+    LLaMA-2-7B shape (16 GiB) out to a 4096-block pinned pool and back into other slots, on
+    side streams, while 8 requests migrate on the main stream.  Checked by the round trip
+    itself (every block that came back equals the block that left), by canaries on host
+    blocks no swap named, and by the oracle on a sample."""
+    w = workloads.config5()
+    shape = w.shape
+    kvm.reset()
+    k_gpu = workloads.fill_uniform(shape.pool_shape(w.gpu_blocks), w.seed, "cuda")
+    v_gpu = workloads.fill_uniform(shape.pool_shape(w.gpu_blocks), w.seed + 500, "cuda")
+    k_ref, v_ref = k_gpu.clone(), v_gpu.clone()
+    k_host = torch.empty(shape.pool_shape(w.host_blocks), dtype=shape.dtype, pin_memory=True)
+    v_host = torch.empty(shape.pool_shape(w.host_blocks), dtype=shape.dtype, pin_memory=True)
+    k_host.view(torch.int16).fill_(workloads.CANARY_BITS)
+    v_host.view(torch.int16).fill_(workloads.CANARY_BITS)
+    mig = w.migrate
+    g = geom_of(mig)
+    src_k = workloads.fill_uniform(mig.src_pool_shape(), 77, "cuda")
+    src_v = workloads.fill_uniform(mig.src_pool_shape(), 78, "cuda")
+    kvm.register_source(1, 1, 0, 0, g.num_layers, g.num_kv_heads, src_k.data_ptr(), src_v.data_ptr(),
+                        src_k.numel() * 2)
+    out_stream, in_stream = torch.cuda.Stream(), torch.cuda.Stream()
+    torch.cuda.synchronize()
+    do_swap(kvm, w.out_gpu_ids, w.out_host_ids, False, k_gpu, v_gpu, k_host, v_host, out_stream)
+    out_done = torch.cuda.Event()
+    out_done.record(out_stream)
+    for call in mig.calls:
+        kvm.migrate(kvm_geom(g), call.ctx_idx, call.dec_idx, k_gpu.data_ptr(), v_gpu.data_ptr(), w.gpu_blocks,
+                    torch.cuda.current_stream().cuda_stream)
+    in_stream.wait_event(out_done)
+    do_swap(kvm, w.out_host_ids, w.in_gpu_ids, True, k_gpu, v_gpu, k_host, v_host, in_stream)
+    torch.cuda.synchronize()
+    for ref, pool in ((k_ref, k_gpu), (v_ref, v_gpu)):
+        for i0 in range(0, len(w.out_gpu_ids), 256):
+            a = torch.tensor(w.out_gpu_ids[i0:i0 + 256], device="cuda")
+            b = torch.tensor(w.in_gpu_ids[i0:i0 + 256], device="cuda")
+            assert torch.equal(pool.view(torch.int16)[b], ref.view(torch.int16)[a])
+    for call in mig.calls:
+        a = torch.tensor(call.ctx_idx, device="cuda")
+        b = torch.tensor(call.dec_idx, device="cuda")
+        assert torch.equal(k_gpu.view(torch.int16)[b], src_k.view(torch.int16)[a])
+        assert torch.equal(v_gpu.view(torch.int16)[b], src_v.view(torch.int16)[a])
+    named = torch.zeros(w.host_blocks, dtype=torch.bool)
+    named[torch.tensor(w.out_host_ids)] = True
+    for b in (~named).nonzero().flatten().tolist()[::64]:
+        assert bool((k_host[b].view(torch.int16) == workloads.CANARY_BITS).all())
+    # oracle on a sample of the swapped blocks: host copy and returned copy
+    pick = list(range(0, len(w.out_gpu_ids), 128))
+    src_ids = [w.out_gpu_ids[i] for i in pick]
+    small_ref = k_ref[torch.tensor(src_ids, device="cuda")].cpu()
+    want_host = canary_pool((len(pick),) + tuple(small_ref.shape[1:]))
+    oracle.swap_c(list(range(len(pick))), list(range(len(pick))), small_ref, want_host)
+    assert same_bits(k_host[torch.tensor([w.out_host_ids[i] for i in pick])], want_host)
+    assert same_bits(k_gpu[torch.tensor([w.in_gpu_ids[i] for i in pick], device="cuda")].cpu(), want_host)
+    kvm.reset()
