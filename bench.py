@@ -252,7 +252,8 @@ def main():
             "bound": "hbm", "achieved": round(bytes_per_launch / (launch_us * 1e-6) / 1e9, 2), "peak": HBM_PEAK_GBPS,
             "unit": "GB/s", "frac": round(bytes_per_launch / (launch_us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
             "traffic": measured_traffic(args.config, bytes_per_launch),
-            "kernel": "kvm_copy_kernel<u32x4>", "launches_per_step": launches_per_step,
+            "kernel": ("kvm_copy_simple_kernel" if plan["simple_kernel"] else "kvm_copy_kernel") + "<u32x4, 64, 1>",
+            "launches_per_step": launches_per_step,
             "avg_launch_us": round(launch_us, 2), "algorithmic_bytes_per_launch": round(bytes_per_launch),
             "workgroups_per_block": plan["workgroups_per_block"], "workgroup_size": plan["threads"],
         },

@@ -165,7 +165,8 @@ def get_option(name: str) -> int:
 
 
 def migrate_plan(g: KvmGeom, n: int, dst_k: int, dst_v: int) -> dict:
-    out = (ctypes.c_int64 * 6)()
+    out = (ctypes.c_int64 * 8)()
     _check(lib.kvm_migrate_plan(ctypes.byref(g), n, dst_k, dst_v, out))
-    keys = ("workgroups_per_block", "threads", "vector_bytes", "segments", "launches", "payload_bytes_per_block")
+    keys = ("workgroups_per_block", "threads", "vector_bytes", "segments", "launches", "payload_bytes_per_block",
+            "simple_kernel")
     return dict(zip(keys, list(out)))

@@ -666,7 +666,7 @@ WalkFn pick_walk(int vec)
 // walk_wgs > 0 selects the link-bound form with that many workgroups per pool kind.
 int launch_copy(std::vector<Seg> segs, const IdxPair *pairs, int64_t n, char *dst_k, char *dst_v,
                 uint64_t dst_block_stride, int vec, hipStream_t stream, int64_t *out_launches,
-                int64_t *out_wgs_per_block, int *out_threads, int walk_wgs = 0)
+                int64_t *out_wgs_per_block, int *out_threads, int walk_wgs = 0, bool *out_simple = nullptr)
 {
     Launch k;
     if (int rc = pick_kernel(vec, &k)) return rc;
@@ -674,6 +674,7 @@ int launch_copy(std::vector<Seg> segs, const IdxPair *pairs, int64_t n, char *ds
     uint32_t tile_bytes = (uint32_t)opt_tile_bytes.load();
     if (tile_bytes == 0) tile_bytes = (uint32_t)((walk_wgs > 0 ? 256 * 4 : k.threads * k.unroll) * vec);
     int64_t launches = 0, wgs_per_block = 0;
+    bool all_simple = true;
     for (size_t s0 = 0; s0 < segs.size(); s0 += kMaxSegs) {
         MigrateArgs args;
         args.dst_k = dst_k;
@@ -691,6 +692,12 @@ int launch_copy(std::vector<Seg> segs, const IdxPair *pairs, int64_t n, char *ds
         }
         for (uint32_t j = args.nseg; j < kMaxSegs; ++j) args.tile_end[j] = UINT32_MAX;
         args.tile_end[args.nseg - 1] = UINT32_MAX;   // nothing lies past the last segment
+        // one collapsed segment of full one-shot tiles takes the short-prologue kernel
+        const Seg &first = args.seg[0];
+        const bool simple = walk_wgs == 0 && k.simple_fn && opt_simple.load() && args.nseg == 1 &&
+                            first.n_rows == 1 && first.rows_per_tile == 1 && first.run_bytes % tile_bytes == 0 &&
+                            tile_bytes == (uint32_t)(k.threads * k.unroll * vec);
+        all_simple = all_simple && simple;
         wgs_per_block += 2 * (int64_t)tiles_total;
         // a launch is a 1-D grid of 2 * tiles * blocks workgroups, which must stay below 2^31
         if (tiles_total == 0 || tiles_total > (1u << 29))
@@ -706,10 +713,6 @@ int launch_copy(std::vector<Seg> segs, const IdxPair *pairs, int64_t n, char *ds
                                        dim3(256), 0, stream, args, tiles_total);
                 } else {
                     plan_work(args, tiles_total, tile_bytes);
-                    const Seg &s0 = args.seg[0];
-                    const bool simple = k.simple_fn && opt_simple.load() && args.nseg == 1 && s0.n_rows == 1 &&
-                                        s0.rows_per_tile == 1 && s0.run_bytes % tile_bytes == 0 &&
-                                        tile_bytes == (uint32_t)(k.threads * k.unroll * vec);
                     hipLaunchKernelGGL(simple ? k.simple_fn : k.fn, dim3(2 * args.work_padded), dim3(k.threads),
                                        (size_t)opt_lds_pad.load(), stream, args);
                 }
@@ -722,6 +725,7 @@ int launch_copy(std::vector<Seg> segs, const IdxPair *pairs, int64_t n, char *ds
     if (out_launches) *out_launches = launches;
     if (out_wgs_per_block) *out_wgs_per_block = wgs_per_block;
     if (out_threads) *out_threads = k.threads;
+    if (out_simple) *out_simple = all_simple && !segs.empty();
     return KVM_OK;
 }
 
@@ -954,15 +958,16 @@ int kvm_reset(void)
     return KVM_OK;
 }
 
-int kvm_migrate_plan(const KvmGeom *geom, int64_t n, const void *dst_k, const void *dst_v, int64_t out[6])
+int kvm_migrate_plan(const KvmGeom *geom, int64_t n, const void *dst_k, const void *dst_v, int64_t out[8])
 {
     if (!out) return fail(KVM_EINVAL, "out is null");
     Plan plan;
     if (int rc = build_plan(geom, dst_k, dst_v, &plan)) return rc;
     int64_t launches = 0, wgs = 0;
     int threads = 0;
+    bool simple = false;
     if (int rc = launch_copy(plan.segs, nullptr, n, nullptr, nullptr, plan.dst_block_stride, plan.vec,
-                             nullptr, &launches, &wgs, &threads))
+                             nullptr, &launches, &wgs, &threads, 0, &simple))
         return rc;
     out[0] = wgs;
     out[1] = threads;
@@ -970,6 +975,8 @@ int kvm_migrate_plan(const KvmGeom *geom, int64_t n, const void *dst_k, const vo
     out[3] = (int64_t)plan.segs.size();
     out[4] = launches;
     out[5] = plan.payload_per_block;
+    out[6] = simple ? 1 : 0;
+    out[7] = 0;
     return KVM_OK;
 }
 

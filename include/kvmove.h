@@ -162,11 +162,12 @@ int64_t kvm_get_option(const char *name);
  * Launch shape kvm_migrate would use for this geometry and n blocks, for tests and
  * reports: out[0] = workgroups per block (K and V together), out[1] = workgroup size,
  * out[2] = vector width in bytes, out[3] = number of source segments,
- * out[4] = kernel launches, out[5] = payload bytes per block (K+V, this rank's share).
+ * out[4] = kernel launches, out[5] = payload bytes per block (K+V, this rank's share),
+ * out[6] = 1 when the short-prologue kernel (kvm_copy_simple_kernel) serves the shape, out[7] = 0.
  * Needs the sources registered (alignment of their bases picks the vector width).
  */
 int kvm_migrate_plan(const KvmGeom *geom, int64_t n, const void *dst_k, const void *dst_v,
-                     int64_t out[6]);
+                     int64_t out[8]);
 
 /*
  * Test hook (no counterpart in the reference): n / d computed the way the kernel computes

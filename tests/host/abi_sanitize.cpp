@@ -74,7 +74,7 @@ int main()
     EXPECT(kvm_migrate(&bad, ci.data(), di.data(), 1, fake_k, fake_v, 8, nullptr) == KVM_EINVAL);
     bad = geom(1 << 20, 1 << 10, 16, 128, 2);                   // a block beyond 4 GiB
     EXPECT(kvm_migrate(&bad, ci.data(), di.data(), 1, fake_k, fake_v, 8, nullptr) == KVM_EINVAL);
-    int64_t plan[6];
+    int64_t plan[8];
     EXPECT(kvm_migrate_plan(&g, 10, fake_k, fake_v, nullptr) == KVM_EINVAL);
     EXPECT(kvm_migrate_plan(&g, 10, fake_k, fake_v, plan) == KVM_ENOTREG);
 
