@@ -627,7 +627,6 @@ int build_plan(const KvmGeom *g, const void *dst_k, const void *dst_v, Plan *pla
     return KVM_OK;
 }
 
-// Enqueues the copy kernel over `segs` x `pairs`, as many launches as the 4 KiB argument needs.
 // Fills the second header record: the id -> work item mapping for `tiles` tiles per block.
 void plan_work(MigrateArgs &args, uint32_t tiles, uint32_t tile_bytes)
 {
@@ -663,7 +662,9 @@ WalkFn pick_walk(int vec)
                      : kvm_walk_kernel<uint8_t>;
 }
 
-// walk_wgs > 0 selects the link-bound form with that many workgroups per pool kind.
+// Enqueues the copy over `segs` x `pairs`, as many launches as the 4 KiB argument needs
+// (8 segments and 432 index pairs each).  `pairs == nullptr` only counts what would be
+// launched.  walk_wgs > 0 selects the link-bound form with that many workgroups per pool kind.
 int launch_copy(std::vector<Seg> segs, const IdxPair *pairs, int64_t n, char *dst_k, char *dst_v,
                 uint64_t dst_block_stride, int vec, hipStream_t stream, int64_t *out_launches,
                 int64_t *out_wgs_per_block, int *out_threads, int walk_wgs = 0, bool *out_simple = nullptr)
@@ -782,7 +783,9 @@ int host_pinned(const void *p, const char *what)
     return KVM_OK;
 }
 
-// Pointers already checked by device_of / host_pinned (the query costs microseconds).
+// Pointers already checked by device_of / host_pinned (the query costs microseconds).  Pools
+// are borrowed for as long as the caller uses them, so a base address keeps its kind;
+// kvm_reset() forgets what was learnt.
 std::mutex g_checked_mu;
 std::map<const void *, int> g_checked;  // ptr -> device, or -1 for pinned host
 
@@ -816,19 +819,21 @@ int checked_pinned(const void *p, const char *what)
 }
 
 // A second stream (default priority) and the two events that fork it from and join it back
-// into the caller's stream; one set per device, made on first use, kept until the process ends.
+// into the caller's stream; one set per device and direction (so that a swap-out and a
+// swap-in issued on different streams still overlap), made on first use, kept until the
+// process ends.
 struct Fork {
     hipStream_t side = nullptr;
     hipEvent_t forked = nullptr, joined = nullptr;
 };
 std::mutex g_fork_mu;
-std::map<int, Fork> g_forks;
+std::map<std::pair<int, bool>, Fork> g_forks;
 
-int get_fork(Fork **out)
+int get_fork(bool is_swap_in, Fork **out)
 {
     int dev = 0;
     KVM_HIP(hipGetDevice(&dev));
-    Fork &f = g_forks[dev];
+    Fork &f = g_forks[{dev, is_swap_in}];
     if (!f.side) {
         KVM_HIP(hipStreamCreateWithFlags(&f.side, hipStreamNonBlocking));
         KVM_HIP(hipEventCreateWithFlags(&f.forked, hipEventDisableTiming));
@@ -987,11 +992,11 @@ int kvm_migrate(const KvmGeom *geom, const int64_t *ctx_idx, const int64_t *dec_
     if (!dst_k || !dst_v) return fail(KVM_EINVAL, "destination pool is null");
     if (dst_num_blocks <= 0) return fail(KVM_EINVAL, "destination pool has no blocks");
     if (n > 0 && (!ctx_idx || !dec_idx)) return fail(KVM_EINVAL, "index list is null");
+    if (n == 0) return check_geom(geom);   // an empty list moves nothing, whatever is registered
     Plan plan;
     if (int rc = build_plan(geom, dst_k, dst_v, &plan)) return rc;
     if (int rc = checked_device(dst_k, "decoding K pool")) return rc;
     if (int rc = checked_device(dst_v, "decoding V pool")) return rc;
-    if (n == 0) return KVM_OK;
     std::vector<IdxPair> pairs;
     if (int rc = check_indices(ctx_idx, dec_idx, n, plan.min_src_blocks, dst_num_blocks,
                                "context_block_indexes", "decoding_block_indexes", &pairs))
@@ -1054,7 +1059,7 @@ int kvm_swap(const int64_t *src_ids, const int64_t *dst_ids, int64_t n, int is_s
     std::unique_lock<std::mutex> fork_lock;
     if (opt_swap_mode.load() == 2) {
         fork_lock = std::unique_lock<std::mutex>(g_fork_mu);
-        if (int rc = get_fork(&fork)) return rc;
+        if (int rc = get_fork(is_swap_in != 0, &fork)) return rc;
         KVM_HIP(hipEventRecord(fork->forked, st));
         KVM_HIP(hipStreamWaitEvent(fork->side, fork->forked, 0));
         st_v = fork->side;

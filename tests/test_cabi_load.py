@@ -51,6 +51,7 @@ def test_argument_errors_need_no_gpu(kvm, fresh_registry):
     with pytest.raises(kvm.KvmError) as e:
         kvm.migrate(g, [0], [0], 4096, 8192, 4)                 # nothing registered
     assert e.value.code == kvm.KVM_ENOTREG
+    kvm.migrate(g, [], [], 4096, 8192, 4)                       # an empty list is a no-op even then
     with pytest.raises(kvm.KvmError) as e:
         kvm.register_mem_handle([0] * 8, [0] * 8, 4, 4, [1, 0, 1, 0], [1, 0, 1, 0])
     assert e.value.code == kvm.KVM_EHANDLE
