@@ -44,7 +44,10 @@ def parse_args():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also time the plain contiguous copy kernel (adds launches to a profile)")
     ap.add_argument("--swap-blocks", type=int, default=0, help="config 5: blocks to swap (default 2048)")
-    ap.add_argument("--swap-wgs", type=int, nargs="*", default=[4],
+    ap.add_argument("--swap-shape", type=str, default="", metavar="L,H,D",
+                    help="config 5: local layers, KV heads and head_dim of the pools instead of the LLaMA-2-7B "
+                         "shape, e.g. 12,12,64 (288 KiB slabs) or 80,2,128 (640 KiB slabs)")
+    ap.add_argument("--swap-wgs", type=int, nargs="*", default=[6],
                     help="config 5: workgroup counts to try for the swap kernel")
     ap.add_argument("--plain-copy-only", type=int, default=0, metavar="MiB",
                     help="launch nothing but plain contiguous copies of this size (counter calibration)")
@@ -277,7 +280,13 @@ def run_swap_bench(args):
     from distserve_amd import cabi, workloads
 
     torch.cuda.set_device(0)
-    w = workloads.config5(swap_blocks=args.swap_blocks) if args.swap_blocks else workloads.config5()
+    kw = {}
+    if args.swap_blocks:
+        kw["swap_blocks"] = args.swap_blocks
+    if args.swap_shape:
+        layers, heads, head_dim = (int(x) for x in args.swap_shape.split(","))
+        kw["shape"] = workloads.KvShape(layers, heads, head_dim)
+    w = workloads.config5(**kw)
     shape = w.shape
     main = torch.cuda.current_stream()
     out_stream, in_stream = torch.cuda.Stream(), torch.cuda.Stream()
@@ -335,7 +344,9 @@ def run_swap_bench(args):
 
     results = {}
     bytes_dir = w.bytes_per_direction
-    default_mode, default_wgs = cabi.get_option("swap_mode"), cabi.get_option("swap_wgs")
+    option_mode, default_wgs = cabi.get_option("swap_mode"), cabi.get_option("swap_wgs")
+    # what the library's default takes for this block list (mode 3 decides per call)
+    default_mode = cabi.swap_plan(w.out_gpu_ids, w.out_host_ids, slab)["mode"]
     if default_mode == 1 and default_wgs not in args.swap_wgs:
         args.swap_wgs.append(default_wgs)
 
@@ -412,7 +423,7 @@ def run_swap_bench(args):
                 row["migration_ms_alone"] = round(migrate_alone_ms, 3)
             rows.append(row)
         results[mode_name] = rows
-    cabi.set_option("swap_mode", default_mode)
+    cabi.set_option("swap_mode", option_mode)
     cabi.set_option("swap_wgs", default_wgs)
     cpu = None
     if not args.no_cpu_baseline:
@@ -423,7 +434,9 @@ def run_swap_bench(args):
     total_s = best["swap_out_ms"] * 1e-3 + best["swap_in_ms"] * 1e-3
     cabi.reset()
     return {
-        "metric": "KV swap GB/s (fraction of measured host link), LLaMA-2-7B shape, overlapped with an 8-request migration",
+        "metric": ("KV swap GB/s (fraction of measured host link), "
+                   + (f"pools of {args.swap_shape} layers,heads,head_dim" if args.swap_shape else "LLaMA-2-7B shape")
+                   + ", overlapped with an 8-request migration"),
         "value": round(2 * bytes_dir / total_s / 1e9, 2), "unit": "GB/s", "n_gpus": 1, "steps": 1, "warmup": 1,
         "ms_per_step": round(total_s * 1e3, 2), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "u8", "data": "synthetic",
@@ -433,6 +446,8 @@ def run_swap_bench(args):
                    "value_counts": "bytes over the host link, swap-out plus swap-in, default swap mode, overlapped run"},
         "link_GBps": {k: round(v, 2) for k, v in link.items()},
         "pin_host_pools_s": round(pin_s, 2),
+        "default_swap_mode": {"option": option_mode, "taken_for_this_workload": default_mode,
+                              "variant": default_name[0] if default_name else None},
         "swap": results,
         "cpu_baseline": cpu,
         "roofline": {"bound": "host link", "achieved": round(2 * bytes_dir / total_s / 1e9, 2),

@@ -24,7 +24,7 @@ KVM_HANDLE_WORDS = 8
 EXPORTS = (
     "kvm_version", "kvm_last_error", "kvm_get_mem_handle", "kvm_register_mem_handle",
     "kvm_register_source", "kvm_reset", "kvm_migrate", "kvm_swap", "kvm_copy_plain",
-    "kvm_set_option", "kvm_get_option", "kvm_migrate_plan", "kvm_debug_divide",
+    "kvm_set_option", "kvm_get_option", "kvm_migrate_plan", "kvm_swap_plan", "kvm_debug_divide",
 )
 
 
@@ -68,6 +68,7 @@ def _load() -> ctypes.CDLL:
     lib.kvm_get_option.argtypes = [ctypes.c_char_p]
     lib.kvm_get_option.restype = i64
     lib.kvm_migrate_plan.argtypes = [ctypes.POINTER(KvmGeom), i64, vp, vp, ip]
+    lib.kvm_swap_plan.argtypes = [ip, ip, i64, i64, ip]
     lib.kvm_debug_divide.argtypes = [ctypes.c_uint32, ctypes.c_uint32]
     lib.kvm_debug_divide.restype = ctypes.c_uint32
     for name in EXPORTS:
@@ -162,6 +163,14 @@ def get_option(name: str) -> int:
     if v == KVM_EINVAL and lib.kvm_last_error():
         raise KvmError(KVM_EINVAL, lib.kvm_last_error().decode())
     return v
+
+
+def swap_plan(src_ids: Sequence[int], dst_ids: Sequence[int], slab_bytes: int) -> dict:
+    if len(src_ids) != len(dst_ids):
+        raise KvmError(KVM_EINVAL, f"{len(src_ids)} source blocks but {len(dst_ids)} target blocks")
+    out = (ctypes.c_int64 * 4)()
+    _check(lib.kvm_swap_plan(_arr(src_ids), _arr(dst_ids), len(src_ids), slab_bytes, out))
+    return dict(zip(("mode", "copies_per_pool", "launches", "workgroups_per_pool_kind"), list(out)))
 
 
 def migrate_plan(g: KvmGeom, n: int, dst_k: int, dst_v: int) -> dict:

@@ -378,8 +378,9 @@ std::atomic<int64_t> opt_threads{64};
 std::atomic<int64_t> opt_unroll{1};
 std::atomic<int64_t> opt_nt_load{1};
 std::atomic<int64_t> opt_nt_store{1};
-std::atomic<int64_t> opt_swap_mode{2};
-std::atomic<int64_t> opt_swap_wgs{4};
+std::atomic<int64_t> opt_swap_mode{3};
+std::atomic<int64_t> opt_swap_wgs{6};
+std::atomic<int64_t> opt_swap_kernel_below{2 << 20};
 std::atomic<int64_t> opt_lds_pad{0};
 std::atomic<int64_t> opt_wave_contig{0};
 std::atomic<int64_t> opt_xcd_map{1};
@@ -395,6 +396,7 @@ std::atomic<int64_t> *find_opt(const char *name)
     if (!strcmp(name, "nt_store")) return &opt_nt_store;
     if (!strcmp(name, "swap_mode")) return &opt_swap_mode;
     if (!strcmp(name, "swap_wgs")) return &opt_swap_wgs;
+    if (!strcmp(name, "swap_kernel_below")) return &opt_swap_kernel_below;
     if (!strcmp(name, "lds_pad")) return &opt_lds_pad;
     if (!strcmp(name, "wave_contig")) return &opt_wave_contig;
     if (!strcmp(name, "xcd_map")) return &opt_xcd_map;
@@ -843,6 +845,21 @@ int get_fork(bool is_swap_in, Fork **out)
     return KVM_OK;
 }
 
+// Which implementation serves a swap call (0, 1 or 2; see the "swap_mode" option).  Mode 3
+// decides per call: a copy engine needs about 2 MiB per copy to hide its per-copy cost
+// (measured: 4 MiB copies reach 98 % of the link, 1 MiB 85-91 %, 288 KiB 55 %, 64 KiB 20 %),
+// the copy kernel does not care (90-99 % at every slab size).  *out_runs = copies per pool.
+int64_t swap_mode_for(const IdxPair *pairs, int64_t n, int64_t slab_bytes, int64_t *out_runs)
+{
+    int64_t runs = n > 0 ? 1 : 0;
+    for (int64_t i = 1; i < n; ++i)
+        runs += !(pairs[i].ctx == pairs[i - 1].ctx + 1 && pairs[i].dec == pairs[i - 1].dec + 1);
+    if (out_runs) *out_runs = runs;
+    const int64_t mode = opt_swap_mode.load();
+    if (mode != 3) return mode;
+    return runs > 0 && (n * slab_bytes) / runs < opt_swap_kernel_below.load() ? 1 : 2;
+}
+
 }  // namespace
 
 // ------------------------------------------------------------------------- C ABI
@@ -864,7 +881,8 @@ int kvm_set_option(const char *name, int64_t value)
     else if (o == &opt_swap_wgs) ok = value >= 1 && value <= 4096;
     else if (o == &opt_lds_pad) ok = value >= 0 && value <= 65536;
     else if (o == &opt_xcd_map) ok = value >= 0 && value <= 3;
-    else if (o == &opt_swap_mode) ok = value >= 0 && value <= 2;
+    else if (o == &opt_swap_mode) ok = value >= 0 && value <= 3;
+    else if (o == &opt_swap_kernel_below) ok = value >= 0 && value <= (1ll << 32);
     else ok = value == 0 || value == 1;
     if (!ok) return fail(KVM_EINVAL, "value %lld is not valid for option '%s'", (long long)value, name);
     o->store(value);
@@ -1005,6 +1023,27 @@ int kvm_migrate(const KvmGeom *geom, const int64_t *ctx_idx, const int64_t *dec_
                        plan.dst_block_stride, plan.vec, (hipStream_t)stream, nullptr, nullptr, nullptr);
 }
 
+int kvm_swap_plan(const int64_t *src_ids, const int64_t *dst_ids, int64_t n, int64_t slab_bytes, int64_t out[4])
+{
+    if (!out) return fail(KVM_EINVAL, "out is null");
+    if (n < 0 || (n > 0 && (!src_ids || !dst_ids))) return fail(KVM_EINVAL, "bad index lists");
+    if (slab_bytes <= 0 || slab_bytes >= (1ll << 32))
+        return fail(KVM_EINVAL, "slab_bytes %lld must be in (0, 4 GiB)", (long long)slab_bytes);
+    std::vector<IdxPair> pairs((size_t)n);
+    for (int64_t i = 0; i < n; ++i) {
+        if (src_ids[i] < 0 || src_ids[i] > INT32_MAX || dst_ids[i] < 0 || dst_ids[i] > INT32_MAX)
+            return fail(KVM_ERANGE, "block id out of range at position %lld", (long long)i);
+        pairs[(size_t)i] = IdxPair{(int32_t)src_ids[i], (int32_t)dst_ids[i]};
+    }
+    int64_t runs = 0;
+    const int64_t mode = swap_mode_for(pairs.data(), n, slab_bytes, &runs);
+    out[0] = mode;
+    out[1] = runs;
+    out[2] = mode == 1 ? (n + kMaxIdx - 1) / kMaxIdx : 0;
+    out[3] = mode == 1 ? opt_swap_wgs.load() : 0;
+    return KVM_OK;
+}
+
 int kvm_swap(const int64_t *src_ids, const int64_t *dst_ids, int64_t n, int is_swap_in, void *k_gpu,
              void *v_gpu, void *k_host, void *v_host, int64_t slab_bytes, int64_t n_gpu_blocks,
              int64_t n_host_blocks, void *stream)
@@ -1031,7 +1070,9 @@ int kvm_swap(const int64_t *src_ids, const int64_t *dst_ids, int64_t n, int is_s
     char *dst_k = (char *)(is_swap_in ? k_gpu : k_host), *dst_v = (char *)(is_swap_in ? v_gpu : v_host);
     hipStream_t st = (hipStream_t)stream;
 
-    if (opt_swap_mode.load() == 1) {
+    const int64_t mode = swap_mode_for(pairs.data(), n, slab_bytes, nullptr);
+
+    if (mode == 1) {
         // One gather launch; the pinned pools are read or written in place over the host link.
         void *dk = nullptr, *dv = nullptr;
         KVM_HIP(hipHostGetDevicePointer(&dk, k_host, 0));
@@ -1057,7 +1098,7 @@ int kvm_swap(const int64_t *src_ids, const int64_t *dst_ids, int64_t n, int is_s
     hipStream_t st_v = st;
     Fork *fork = nullptr;
     std::unique_lock<std::mutex> fork_lock;
-    if (opt_swap_mode.load() == 2) {
+    if (mode == 2) {
         fork_lock = std::unique_lock<std::mutex>(g_fork_mu);
         if (int rc = get_fork(is_swap_in != 0, &fork)) return rc;
         KVM_HIP(hipEventRecord(fork->forked, st));

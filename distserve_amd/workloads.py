@@ -242,7 +242,9 @@ def config5(seed: int = 5, gpu_blocks: int = 4096, host_blocks: int = 4096, swap
         assert at + n <= migrate_src_blocks, "migration source pool too small"
         mig.calls.append(MigrateCall(rid, length, src_perm[at:at + n], mig_targets[at:at + n]))
         at += n
-    return SwapWorkload("cfg5-swap-llama2-7b", shape, gpu_blocks, host_blocks, seed, out_gpu, host_ids,
+    name = "cfg5-swap-llama2-7b" if shape == KvShape(32, 32, 128) else (
+        f"cfg5-swap-{shape.num_layers}x{shape.num_kv_heads}x{shape.head_dim}")
+    return SwapWorkload(name, shape, gpu_blocks, host_blocks, seed, out_gpu, host_ids,
                         in_gpu, mig)
 
 

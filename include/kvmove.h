@@ -147,12 +147,17 @@ int kvm_copy_plain(void *dst, const void *src, int64_t nbytes, void *stream);
  *                    reports KVM_EINVAL for one that is not)
  *   "nt_load"        1 = nontemporal loads, 0 = plain
  *   "nt_store"       1 = nontemporal stores, 0 = plain
- *   "swap_mode"      2 (default) = hipMemcpyAsync per contiguous run, K pool on the caller's
- *                    stream and V pool on a second stream forked from and joined back into it,
+ *   "swap_mode"      3 (default) = chosen per call: mode 2 when the copies of the call average
+ *                        at least "swap_kernel_below" bytes each, else mode 1,
+ *                    2 = hipMemcpyAsync per run of blocks consecutive on both sides, K pool on
+ *                        the caller's stream and V pool on a second stream forked from and
+ *                        joined back into it,
  *                    0 = the same with both pools on the caller's stream,
- *                    1 = copy kernel that reads/writes the pinned pools in place (fast alone,
- *                        but it slows HBM-bound kernels that run beside it)
- *   "swap_wgs"       workgroups per pool kind of the swap kernel (mode 1), 1..4096
+ *                    1 = copy kernel that reads/writes the pinned pools in place: one launch
+ *                        per 432 blocks whatever their size, a few microseconds of host time
+ *   "swap_wgs"       workgroups per pool kind of the swap kernel, 1..4096 (default 6; from
+ *                    about 12 on the kernel slows HBM-bound kernels that run beside it)
+ *   "swap_kernel_below"  bytes per copy under which mode 3 takes the kernel (default 2 MiB)
  * kvm_get_option returns the value or KVM_EINVAL (as int64) for an unknown name.
  */
 int kvm_set_option(const char *name, int64_t value);
@@ -168,6 +173,16 @@ int64_t kvm_get_option(const char *name);
  */
 int kvm_migrate_plan(const KvmGeom *geom, int64_t n, const void *dst_k, const void *dst_v,
                      int64_t out[8]);
+
+/*
+ * How kvm_swap would serve these lists at this slab size under the current options, for
+ * tests and reports (no counterpart in the reference): out[0] = implementation taken (0, 1
+ * or 2, as "swap_mode" numbers them), out[1] = copies per pool = runs of blocks consecutive
+ * on both sides, out[2] = kernel launches (mode 1, else 0), out[3] = workgroups per pool
+ * kind of each launch (mode 1, else 0).  Touches no device and no pool.
+ */
+int kvm_swap_plan(const int64_t *src_ids, const int64_t *dst_ids, int64_t n, int64_t slab_bytes,
+                  int64_t out[4]);
 
 /*
  * Test hook (no counterpart in the reference): n / d computed the way the kernel computes

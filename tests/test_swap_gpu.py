@@ -14,7 +14,7 @@ pytestmark = pytest.mark.gpu
 BLOCK = (3, 4, 16, 32)          # layers, heads, block_size, head_dim -> 12 KiB slabs
 
 
-@pytest.fixture(params=[0, 1, 2], ids=["memcpy", "kernel", "memcpy-forked"])
+@pytest.fixture(params=[0, 1, 2, 3], ids=["memcpy", "kernel", "memcpy-forked", "auto"])
 def swap_mode(kvm, request):
     old = kvm.get_option("swap_mode")
     kvm.set_option("swap_mode", request.param)
