@@ -46,6 +46,24 @@ def test_every_layout_and_every_decoding_rank(kvm, cpp, ctp, dpp, dtp):
             check_case(kvm, g, 5, 6, ci, di, seed=7)
 
 
+def _uneven_layouts(count=48, seed=5):
+    import random
+    rng = random.Random(seed)
+    every = [c for c in itertools.product((1, 2, 3, 4, 6), repeat=4) if 3 in c or 6 in c]
+    return sorted(rng.sample(every, count))
+
+
+@pytest.mark.parametrize("cpp,ctp,dpp,dtp", _uneven_layouts())
+def test_layouts_whose_splits_do_not_nest(kvm, cpp, ctp, dpp, dtp):
+    """12 layers and 12 heads split by 3 against 2, 4 against 6, ...: a decoding rank overlaps
+    some context ranks only partly, so one call has segments of different widths."""
+    ci, di = [3, 0, 4, 3], [1, 5, 2, 0]
+    for q in range(dpp):
+        for u in range(dtp):
+            g = oracle.Geom(12, 12, 4, 8, 2, cpp, ctp, dpp, dtp, q, u)
+            check_case(kvm, g, 5, 6, ci, di, seed=17)
+
+
 def test_golden_fixtures(kvm):
     import hashlib
     from golden.make_golden import build_case

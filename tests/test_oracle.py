@@ -42,6 +42,28 @@ def test_three_formulations_agree_on_every_layout(cpp, ctp, dpp, dtp):
             assert same_bits(a, b) and same_bits(a, c)
 
 
+def _uneven_layouts(count=40, seed=3):
+    """Layouts over 12 layers and 12 heads in which the two instances' splits do not nest
+    (3 against 2, 4 against 6, ...): a decoding rank then overlaps context ranks partly."""
+    import random
+    rng = random.Random(seed)
+    every = [c for c in itertools.product((1, 2, 3, 4, 6), repeat=4) if 3 in c or 6 in c]
+    return sorted(rng.sample(every, count))
+
+
+@pytest.mark.parametrize("cpp,ctp,dpp,dtp", _uneven_layouts())
+def test_three_formulations_agree_when_the_splits_do_not_nest(cpp, ctp, dpp, dtp):
+    ci, di = [2, 0], [1, 3]
+    for q in range(dpp):
+        for u in range(dtp):
+            g = oracle.Geom(12, 12, 2, 2, 2, cpp, ctp, dpp, dtp, q, u)
+            src = make_src_pools(g, 3, seed=13)
+            a = _run(oracle.migrate_c, g, src, ci, di, 4)
+            b = _run(oracle.migrate_cat, g, src, ci, di, 4)
+            c = _run(oracle.migrate_push_loops, g, src, ci, di, 4)
+            assert same_bits(a, b) and same_bits(a, c)
+
+
 def test_tp1_pp1_reduces_to_index_copy_of_index_select():
     g = oracle.Geom(3, 5, 4, 8, 2)
     src = make_src_pools(g, 9, seed=3)
