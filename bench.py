@@ -216,6 +216,15 @@ def main():
     elapsed_ms = start.elapsed_time(stop)
     ms_per_step = elapsed_ms / args.steps
 
+    # a second pass with an event between steps, for the spread (median and best step)
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
+    marks[0].record(stream)
+    for i in range(args.steps):
+        step()
+        marks[i + 1].record(stream)
+    torch.cuda.synchronize()
+    per_step_ms = sorted(marks[i].elapsed_time(marks[i + 1]) for i in range(args.steps))
+
     payload = w.payload_bytes                       # bytes the decoding rank receives per step
     hbm_bytes = 2 * payload                         # each byte read once and written once
     hbm_gbps = hbm_bytes / (ms_per_step * 1e-3) / 1e9
@@ -245,6 +254,7 @@ def main():
             "value_counts": "HBM bytes read + written (2 x payload) per second",
             "tuning": {k: cabi.get_option(k) for k in ("tile_bytes", "threads", "unroll", "nt_load", "nt_store")},
         },
+        "ms_per_step_median": round(per_step_ms[len(per_step_ms) // 2], 4), "ms_per_step_min": round(per_step_ms[0], 4),
         "payload_GBps": round(payload / (ms_per_step * 1e-3) / 1e9, 2),
         "frac_of_hbm_peak": round(hbm_gbps / HBM_PEAK_GBPS, 4),
         "us_per_request": round(ms_per_step * 1e3 / len(w.calls), 2),
