@@ -453,3 +453,47 @@ def test_every_id_to_work_mapping_copies_the_same_bytes(kvm, xcd_map, simple):
     finally:
         for k, v in saved.items():
             kvm.set_option(k, v)
+
+
+def test_random_geometries_pools_lists_and_tunings(kvm):
+    """300 seeded draws of everything at once: layer/head counts and splits (nesting or not),
+    block and head sizes down to one element, 1/2/4-byte elements, pool sizes, index lists
+    with repeated sources, and every compiled tuning choice."""
+    import random
+
+    rng = random.Random(20)
+    names = ("threads", "unroll", "nt_load", "nt_store", "wave_contig", "tile_bytes", "xcd_map", "simple")
+    saved = {k: kvm.get_option(k) for k in names}
+    flavours = [(64, 1, 1, 1, 0), (64, 2, 1, 1, 0), (128, 1, 1, 1, 0), (256, 1, 1, 1, 0), (256, 4, 1, 1, 0),
+                (256, 8, 1, 1, 0), (512, 2, 1, 1, 0), (512, 8, 1, 1, 0), (1024, 4, 1, 1, 0), (64, 1, 0, 0, 0),
+                (256, 4, 0, 0, 0), (512, 8, 0, 0, 0), (64, 4, 1, 1, 1), (256, 8, 1, 1, 1)]
+    dtypes = {1: torch.uint8, 2: torch.float16, 4: torch.float32}
+
+    def divisors(n):
+        return [d for d in range(1, n + 1) if n % d == 0]
+
+    try:
+        for case in range(300):
+            L, H = rng.choice([1, 2, 3, 4, 6, 8, 12]), rng.choice([1, 2, 3, 4, 6, 8, 12])
+            cpp, dpp = rng.choice(divisors(L)), rng.choice(divisors(L))
+            ctp, dtp = rng.choice(divisors(H)), rng.choice(divisors(H))
+            B, D = rng.choice([1, 2, 3, 4, 8, 16, 32]), rng.choice([1, 2, 3, 5, 8, 16, 40, 64, 80, 128])
+            s = rng.choice([1, 2, 2, 2, 4])
+            g = oracle.Geom(L, H, B, D, s, cpp, ctp, dpp, dtp, rng.randrange(dpp), rng.randrange(dtp))
+            nb_src, nb_dst = rng.randint(1, 12), rng.randint(1, 12)
+            n = rng.randint(0, nb_dst)
+            ci = [rng.randrange(nb_src) for _ in range(n)]
+            di = rng.sample(range(nb_dst), n)
+            threads, unroll, nt_load, nt_store, wave_contig = rng.choice(flavours)
+            chosen = dict(threads=threads, unroll=unroll, nt_load=nt_load, nt_store=nt_store, wave_contig=wave_contig,
+                          tile_bytes=rng.choice([0, 0, 0, 1024, 4096, 16384, 65536]), xcd_map=rng.randrange(4),
+                          simple=rng.randrange(2))
+            for k, v in chosen.items():
+                kvm.set_option(k, v)
+            try:
+                check_case(kvm, g, nb_src, nb_dst, ci, di, seed=case + 1, dtype=dtypes[s])
+            except AssertionError as e:
+                raise AssertionError(f"case {case}: {g} {chosen} ctx {ci} dec {di}: {e}") from None
+    finally:
+        for k, v in saved.items():
+            kvm.set_option(k, v)
