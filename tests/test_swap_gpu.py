@@ -199,3 +199,35 @@ def test_config5_full_size_round_trip_beside_a_migration(kvm):
     assert same_bits(k_host[torch.tensor([w.out_host_ids[i] for i in pick])], want_host)
     assert same_bits(k_gpu[torch.tensor([w.in_gpu_ids[i] for i in pick], device="cuda")].cpu(), want_host)
     kvm.reset()
+
+
+def test_random_slab_sizes_lists_and_pool_sizes(kvm, swap_mode):
+    """60 seeded draws per implementation: slabs from 2 bytes (2-byte vectors in the kernel)
+    to 160 KiB, lists with runs of consecutive blocks, out and back into other slots."""
+    import random
+
+    rng = random.Random(50 + swap_mode)
+    for case in range(60):
+        block = (rng.choice([1, 2, 5]), rng.choice([1, 3, 4]), rng.choice([1, 2, 16]), rng.choice([1, 3, 8, 40, 128]))
+        n_gpu, n_host = rng.randint(2, 14), rng.randint(1, 14)
+        k_gpu, v_gpu, k_host, v_host = pools(n_gpu, n_host, seed=100 + case, block=block)
+        k0, v0 = k_gpu.cpu(), v_gpu.cpu()
+        n = rng.randint(0, min(n_gpu, n_host))
+        if rng.random() < 0.5:                       # a run of consecutive blocks on both sides
+            a, b = rng.randint(0, n_gpu - n), rng.randint(0, n_host - n)
+            out_src, out_dst = list(range(a, a + n)), list(range(b, b + n))
+        else:
+            out_src, out_dst = rng.sample(range(n_gpu), n), rng.sample(range(n_host), n)
+        do_swap(kvm, out_src, out_dst, False, k_gpu, v_gpu, k_host, v_host)
+        torch.cuda.synchronize()
+        want_k, want_v = canary_pool(k_host.shape), canary_pool(v_host.shape)
+        oracle.swap_c(out_src, out_dst, k0, want_k)
+        oracle.swap_c(out_src, out_dst, v0, want_v)
+        assert same_bits(k_host, want_k) and same_bits(v_host, want_v), (case, block, out_src, out_dst)
+        in_dst = rng.sample(range(n_gpu), n)
+        do_swap(kvm, out_dst, in_dst, True, k_gpu, v_gpu, k_host, v_host)
+        torch.cuda.synchronize()
+        exp_k, exp_v = k0.clone(), v0.clone()
+        oracle.swap_c(out_dst, in_dst, want_k, exp_k)
+        oracle.swap_c(out_dst, in_dst, want_v, exp_v)
+        assert same_bits(k_gpu.cpu(), exp_k) and same_bits(v_gpu.cpu(), exp_v), (case, block, out_dst, in_dst)
