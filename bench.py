@@ -47,8 +47,8 @@ def parse_args():
     ap.add_argument("--swap-shape", type=str, default="", metavar="L,H,D",
                     help="config 5: local layers, KV heads and head_dim of the pools instead of the LLaMA-2-7B "
                          "shape, e.g. 12,12,64 (288 KiB slabs) or 80,2,128 (640 KiB slabs)")
-    ap.add_argument("--swap-wgs", type=int, nargs="*", default=[6],
-                    help="config 5: workgroup counts to try for the swap kernel")
+    ap.add_argument("--swap-wgs", type=int, nargs="*", default=None,
+                    help="config 5: workgroup counts to try for the swap kernel (default: the library's)")
     ap.add_argument("--plain-copy-only", type=int, default=0, metavar="MiB",
                     help="launch nothing but plain contiguous copies of this size (counter calibration)")
     return ap.parse_args()
@@ -284,7 +284,9 @@ def run_swap_bench(args):
     """Configuration 5: swap 2048 blocks (16 GiB) from HBM to a pinned host pool and back into
     other GPU slots, on side streams, while an 8-request migration runs on the main stream.
     The denominator is the host link measured in the same run with one large pinned copy per
-    direction.  A step is one swap-out plus one swap-in of the whole block list."""
+    direction.  A step is one swap-out plus one swap-in of the whole block list.  Every
+    implementation is timed three times: alone, beside the 8-request migration (the headline
+    row), and beside migrations issued back to back for as long as both swaps take."""
     import torch
 
     from distserve_amd import cabi, workloads
@@ -355,6 +357,8 @@ def run_swap_bench(args):
     results = {}
     bytes_dir = w.bytes_per_direction
     option_mode, default_wgs = cabi.get_option("swap_mode"), cabi.get_option("swap_wgs")
+    if args.swap_wgs is None:
+        args.swap_wgs = [default_wgs]
     # what the library's default takes for this block list (mode 3 decides per call)
     default_mode = cabi.swap_plan(w.out_gpu_ids, w.out_host_ids, slab)["mode"]
     if default_mode == 1 and default_wgs not in args.swap_wgs:
@@ -384,7 +388,8 @@ def run_swap_bench(args):
         if wgs:
             cabi.set_option("swap_wgs", wgs)
         rows = []
-        for overlapped in (False, True):
+        for phase in ("alone", "overlapped", "busy"):
+            overlapped = phase != "alone"
             k_gpu.copy_(k_ref)
             v_gpu.copy_(v_ref)
             torch.cuda.synchronize()
@@ -395,17 +400,26 @@ def run_swap_bench(args):
             e[1].record(out_stream)
             host_out_us = (time.perf_counter() - t_host) * 1e6
             mig_ms = []
-            if overlapped:
+            if phase == "overlapped":
                 m = [migrate_timed() for _ in range(3)]     # while the swap-out is in flight
             in_stream.wait_event(e[1])        # swap-in reuses slots the swap-out frees
             e[2].record(in_stream)
             swap_in()
             e[3].record(in_stream)
-            if overlapped:
+            if phase == "overlapped":
                 main.wait_event(e[2])                       # start beside the swap-in
                 m += [migrate_timed() for _ in range(3)]
+            if phase == "busy":
+                # migrations back to back on the main stream for longer than both swaps take:
+                # the swap competes with kernels that saturate HBM for all of its duration
+                n_busy = int(1.15 * (rows[0]["swap_out_ms"] + rows[0]["swap_in_ms"]) / migrate_alone_ms) + 1
+                b0, b1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                b0.record(main)
+                for _ in range(n_busy):
+                    migrate_once()
+                b1.record(main)
             torch.cuda.synchronize()
-            if overlapped:
+            if phase == "overlapped":
                 mig_ms = [round(a.elapsed_time(b), 3) for a, b in m]
             t_out, t_in = e[0].elapsed_time(e[1]) * 1e-3, e[2].elapsed_time(e[3]) * 1e-3
             ok = True
@@ -427,9 +441,13 @@ def run_swap_bench(args):
                    "swap_in_frac_of_link": round(bytes_dir / t_in / 1e9 / link["h2d"], 4),
                    "swap_out_ms": round(t_out * 1e3, 2), "swap_in_ms": round(t_in * 1e3, 2),
                    "host_enqueue_swap_out_us": round(host_out_us, 1), "round_trip_bit_exact": ok}
-            if overlapped:
+            if phase == "overlapped":
                 row["migration_ms_beside_swap_out"] = mig_ms[:3]
                 row["migration_ms_beside_swap_in"] = mig_ms[3:]
+                row["migration_ms_alone"] = round(migrate_alone_ms, 3)
+            if phase == "busy":
+                row["continuous_migration"] = True
+                row["migration_ms_avg_of_continuous"] = round(b0.elapsed_time(b1) / n_busy, 3)
                 row["migration_ms_alone"] = round(migrate_alone_ms, 3)
             rows.append(row)
         results[mode_name] = rows

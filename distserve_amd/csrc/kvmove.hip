@@ -379,7 +379,7 @@ std::atomic<int64_t> opt_unroll{1};
 std::atomic<int64_t> opt_nt_load{1};
 std::atomic<int64_t> opt_nt_store{1};
 std::atomic<int64_t> opt_swap_mode{3};
-std::atomic<int64_t> opt_swap_wgs{6};
+std::atomic<int64_t> opt_swap_wgs{8};
 std::atomic<int64_t> opt_swap_kernel_below{2 << 20};
 std::atomic<int64_t> opt_lds_pad{0};
 std::atomic<int64_t> opt_wave_contig{0};

@@ -155,8 +155,10 @@ int kvm_copy_plain(void *dst, const void *src, int64_t nbytes, void *stream);
  *                    0 = the same with both pools on the caller's stream,
  *                    1 = copy kernel that reads/writes the pinned pools in place: one launch
  *                        per 432 blocks whatever their size, a few microseconds of host time
- *   "swap_wgs"       workgroups per pool kind of the swap kernel, 1..4096 (default 6; from
- *                    about 12 on the kernel slows HBM-bound kernels that run beside it)
+ *   "swap_wgs"       workgroups per pool kind of the swap kernel, 1..4096.  Default 8: 99 % of
+ *                    the link on an idle GPU and 87-96 % while other kernels saturate HBM;
+ *                    10-12 hold 96-98 % under such load but slow short kernels beside them,
+ *                    32 and more slow every HBM-bound kernel several times over
  *   "swap_kernel_below"  bytes per copy under which mode 3 takes the kernel (default 2 MiB)
  * kvm_get_option returns the value or KVM_EINVAL (as int64) for an unknown name.
  */
