@@ -6,7 +6,7 @@ from typing import List
 import torch
 
 import oracle
-from distserve_amd.workloads import CANARY_BITS, KvShape, MigrateWorkload
+from distserve_amd.workloads import CANARY_BITS, MigrateWorkload
 
 
 def geom_of(w: MigrateWorkload, dec_pp_rank=None, dec_tp_rank=None) -> oracle.Geom:

@@ -7,8 +7,7 @@ import pytest
 
 from distserve_amd.block_manager import BlockLocation, BlockManager
 from distserve_amd.config import CacheConfig, ModelConfig, ParallelConfig
-from distserve_amd.decoding_stage_scheduler import (DecodingStageFCFSScheduler, DecodingStageSchedConfig,
-                                                   get_decoding_stage_scheduler)
+from distserve_amd.decoding_stage_scheduler import DecodingStageSchedConfig, get_decoding_stage_scheduler
 from distserve_amd.request import MigratingRequest, create_request
 from distserve_amd.utils import Stage
 

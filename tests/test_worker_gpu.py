@@ -4,7 +4,6 @@ import pytest
 import torch
 
 import oracle
-import distserve_amd
 from distserve_amd import (BlockManager, CacheConfig, ContextStageLLMEngine, DecodingStageLLMEngine, ModelConfig,
                            ParallelConfig, Worker, create_request)
 from distserve_amd.utils import Stage
