@@ -785,38 +785,60 @@ int host_pinned(const void *p, const char *what)
     return KVM_OK;
 }
 
-// Pointers already checked by device_of / host_pinned (the query costs microseconds).  Pools
-// are borrowed for as long as the caller uses them, so a base address keeps its kind;
-// kvm_reset() forgets what was learnt.
-std::mutex g_checked_mu;
-std::map<const void *, int> g_checked;  // ptr -> device, or -1 for pinned host
-
-int checked_device(const void *p, const char *what)
+// Bytes from p to the end of the allocation that holds it, 0 when the runtime cannot tell
+// (memory it did not allocate as one range).  A pool that claims more than this would send
+// a kernel past mapped memory, so callers refuse it on the host.
+uint64_t extent_of(const void *p)
 {
-    {
-        std::lock_guard<std::mutex> lock(g_checked_mu);
-        auto it = g_checked.find(p);
-        if (it != g_checked.end() && it->second >= 0) return KVM_OK;
+    hipDeviceptr_t base = nullptr;
+    size_t size = 0;
+    if (hipMemGetAddressRange(&base, &size, (hipDeviceptr_t)p) != hipSuccess || !base) {
+        (void)hipGetLastError();
+        return 0;
     }
-    int dev = 0;
-    if (int rc = device_of(p, what, &dev)) return rc;
-    std::lock_guard<std::mutex> lock(g_checked_mu);
-    if (g_checked.size() > 64) g_checked.clear();
-    g_checked[p] = dev;
+    const char *end = (const char *)base + size;
+    return end > (const char *)p ? (uint64_t)(end - (const char *)p) : 0;
+}
+
+int check_extent(const void *p, uint64_t need, uint64_t extent, const char *what)
+{
+    if (extent != 0 && need > extent)
+        return fail(KVM_ERANGE, "%s (%p) is said to hold %llu bytes but its allocation ends after %llu", what, p,
+                    (unsigned long long)need, (unsigned long long)extent);
     return KVM_OK;
 }
 
-int checked_pinned(const void *p, const char *what)
+// Pointers already checked by device_of / host_pinned (the queries cost microseconds).  Pools
+// are borrowed for as long as the caller uses them, so a base address keeps its kind and its
+// extent; a size that does not fit the remembered extent is looked up afresh before it is
+// refused (the address may belong to a newer allocation), and kvm_reset() forgets everything.
+struct Known {
+    int device;        // -1 for pinned host memory
+    uint64_t extent;   // see extent_of
+};
+std::mutex g_checked_mu;
+std::map<const void *, Known> g_checked;
+
+int checked_pool(const void *p, uint64_t need, bool on_device, const char *what)
 {
     {
         std::lock_guard<std::mutex> lock(g_checked_mu);
         auto it = g_checked.find(p);
-        if (it != g_checked.end() && it->second == -1) return KVM_OK;
+        if (it != g_checked.end() && (it->second.device >= 0) == on_device &&
+            (it->second.extent == 0 || need <= it->second.extent))
+            return KVM_OK;
     }
-    if (int rc = host_pinned(p, what)) return rc;
+    int dev = -1;
+    if (on_device) {
+        if (int rc = device_of(p, what, &dev)) return rc;
+    } else {
+        if (int rc = host_pinned(p, what)) return rc;
+    }
+    const uint64_t extent = extent_of(p);
+    if (int rc = check_extent(p, need, extent, what)) return rc;
     std::lock_guard<std::mutex> lock(g_checked_mu);
     if (g_checked.size() > 64) g_checked.clear();
-    g_checked[p] = -1;
+    g_checked[p] = Known{dev, extent};
     return KVM_OK;
 }
 
@@ -943,6 +965,8 @@ int kvm_register_source(int32_t ctx_pp_size, int32_t ctx_tp_size, int32_t pp_ran
     if (int rc = device_of(k_base, "context K pool", &dk)) return rc;
     if (int rc = device_of(v_base, "context V pool", &dv)) return rc;
     if (dk != dv) return fail(KVM_EINVAL, "context K and V pools sit on different devices");
+    if (int rc = check_extent(k_base, (uint64_t)nbytes_each, extent_of(k_base), "context K pool")) return rc;
+    if (int rc = check_extent(v_base, (uint64_t)nbytes_each, extent_of(v_base), "context V pool")) return rc;
     Source s{ctx_pp_size, ctx_tp_size, num_layers, num_kv_heads, (const char *)k_base,
              (const char *)v_base, nbytes_each};
     std::lock_guard<std::mutex> lock(g_mu);
@@ -1013,8 +1037,9 @@ int kvm_migrate(const KvmGeom *geom, const int64_t *ctx_idx, const int64_t *dec_
     if (n == 0) return check_geom(geom);   // an empty list moves nothing, whatever is registered
     Plan plan;
     if (int rc = build_plan(geom, dst_k, dst_v, &plan)) return rc;
-    if (int rc = checked_device(dst_k, "decoding K pool")) return rc;
-    if (int rc = checked_device(dst_v, "decoding V pool")) return rc;
+    const uint64_t dst_bytes = (uint64_t)dst_num_blocks * plan.dst_block_stride;
+    if (int rc = checked_pool(dst_k, dst_bytes, true, "decoding K pool")) return rc;
+    if (int rc = checked_pool(dst_v, dst_bytes, true, "decoding V pool")) return rc;
     std::vector<IdxPair> pairs;
     if (int rc = check_indices(ctx_idx, dec_idx, n, plan.min_src_blocks, dst_num_blocks,
                                "context_block_indexes", "decoding_block_indexes", &pairs))
@@ -1054,10 +1079,12 @@ int kvm_swap(const int64_t *src_ids, const int64_t *dst_ids, int64_t n, int is_s
         return fail(KVM_EINVAL, "slab_bytes %lld must be in (0, 4 GiB)", (long long)slab_bytes);
     if (n_gpu_blocks <= 0 || n_host_blocks <= 0) return fail(KVM_EINVAL, "a pool has no blocks");
     if (n > 0 && (!src_ids || !dst_ids)) return fail(KVM_EINVAL, "index list is null");
-    if (int rc = checked_device(k_gpu, "GPU K pool")) return rc;
-    if (int rc = checked_device(v_gpu, "GPU V pool")) return rc;
-    if (int rc = checked_pinned(k_host, "host K pool")) return rc;
-    if (int rc = checked_pinned(v_host, "host V pool")) return rc;
+    const uint64_t gpu_bytes = (uint64_t)n_gpu_blocks * (uint64_t)slab_bytes;
+    const uint64_t host_bytes = (uint64_t)n_host_blocks * (uint64_t)slab_bytes;
+    if (int rc = checked_pool(k_gpu, gpu_bytes, true, "GPU K pool")) return rc;
+    if (int rc = checked_pool(v_gpu, gpu_bytes, true, "GPU V pool")) return rc;
+    if (int rc = checked_pool(k_host, host_bytes, false, "host K pool")) return rc;
+    if (int rc = checked_pool(v_host, host_bytes, false, "host V pool")) return rc;
     if (n == 0) return KVM_OK;
 
     const int64_t n_src = is_swap_in ? n_host_blocks : n_gpu_blocks;
@@ -1137,6 +1164,8 @@ int kvm_copy_plain(void *dst, const void *src, int64_t nbytes, void *stream)
 {
     if (!dst || !src || nbytes < 0) return fail(KVM_EINVAL, "kvm_copy_plain: null pointer or negative size");
     if (nbytes == 0) return KVM_OK;
+    if (int rc = checked_pool(dst, (uint64_t)nbytes, true, "kvm_copy_plain destination")) return rc;
+    if (int rc = checked_pool(src, (uint64_t)nbytes, true, "kvm_copy_plain source")) return rc;
     // Expressed as one segment over 4 MiB "blocks" with identity index pairs; K and V
     // stand for the two halves of the buffer, as they stand for the two pools elsewhere.
     const int64_t chunk = 4ll << 20;

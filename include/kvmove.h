@@ -35,7 +35,7 @@ extern "C" {
 
 #define KVM_OK 0
 #define KVM_EINVAL (-1)     /* malformed argument (null pointer, bad size, bad geometry) */
-#define KVM_ERANGE (-2)     /* a block index is outside its pool */
+#define KVM_ERANGE (-2)     /* a block index is outside its pool, or a pool outside its allocation */
 #define KVM_EDUP (-3)       /* a destination block index occurs twice in one call */
 #define KVM_ENOTREG (-4)    /* a context rank the copy needs was never registered */
 #define KVM_EHIP (-5)       /* a HIP runtime call failed */

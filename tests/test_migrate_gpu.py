@@ -497,3 +497,32 @@ def test_random_geometries_pools_lists_and_tunings(kvm):
     finally:
         for k, v in saved.items():
             kvm.set_option(k, v)
+
+
+def test_a_pool_that_claims_more_than_its_allocation_is_refused_on_the_host(kvm):
+    """A wrong block count would send the kernel past mapped memory.  The library asks the
+    runtime where the allocation ends and refuses before anything is launched."""
+    g = oracle.Geom(2, 4, 16, 64, 2)
+    kvm.reset()
+    block_bytes = 2 * 4 * 16 * 64 * 2                       # 16 KiB per block and pool kind
+    nb = 4096                                               # 64 MiB pools: allocations of their own
+    src_k = torch.zeros(g.ctx_pool_shape(nb), dtype=torch.float16, device="cuda")
+    src_v = torch.zeros_like(src_k)
+    dst_k = canary_pool(g.dec_pool_shape(nb)).cuda()
+    dst_v = canary_pool(g.dec_pool_shape(nb)).cuda()
+    with pytest.raises(kvm.KvmError) as e:                   # source said to be 64 times its size
+        kvm.register_source(1, 1, 0, 0, g.num_layers, g.num_kv_heads, src_k.data_ptr(), src_v.data_ptr(),
+                            64 * nb * block_bytes)
+    assert e.value.code == kvm.KVM_ERANGE and "allocation ends" in str(e.value)
+    kvm.register_source(1, 1, 0, 0, g.num_layers, g.num_kv_heads, src_k.data_ptr(), src_v.data_ptr(), nb * block_bytes)
+    s = stream_handle()
+    kvm.migrate(kvm_geom(g), [1], [2], dst_k.data_ptr(), dst_v.data_ptr(), nb, s)      # the true size is fine
+    with pytest.raises(kvm.KvmError) as e:                   # destination said to hold 64 times its blocks
+        kvm.migrate(kvm_geom(g), [1], [3], dst_k.data_ptr(), dst_v.data_ptr(), 64 * nb, s)
+    assert e.value.code == kvm.KVM_ERANGE
+    torch.cuda.synchronize()
+    assert same_bits(dst_k[3].cpu(), canary_pool(g.dec_pool_shape(1))[0])               # nothing was launched
+    kvm.migrate(kvm_geom(g), [1], [3], dst_k.data_ptr(), dst_v.data_ptr(), nb, s)      # and the pool is still usable
+    torch.cuda.synchronize()
+    assert same_bits(dst_k[3].cpu(), src_k[1].cpu())
+    kvm.reset()

@@ -231,3 +231,19 @@ def test_random_slab_sizes_lists_and_pool_sizes(kvm, swap_mode):
         oracle.swap_c(out_dst, in_dst, want_k, exp_k)
         oracle.swap_c(out_dst, in_dst, want_v, exp_v)
         assert same_bits(k_gpu.cpu(), exp_k) and same_bits(v_gpu.cpu(), exp_v), (case, block, out_dst, in_dst)
+
+
+def test_swap_pools_that_claim_more_than_their_allocation_are_refused(kvm, swap_mode):
+    block = (8, 8, 16, 128)                                  # 256 KiB slabs, 64 MiB pools
+    k_gpu, v_gpu, k_host, v_host = pools(256, 256, seed=2, block=block)
+    slab = k_gpu[0].numel() * 2
+    s = torch.cuda.current_stream().cuda_stream
+    ptrs = (k_gpu.data_ptr(), v_gpu.data_ptr(), k_host.data_ptr(), v_host.data_ptr())
+    with pytest.raises(kvm.KvmError) as e:
+        kvm.swap([1], [2], False, *ptrs, slab, 64 * 256, 256, s)          # GPU pool said to be 64 times its size
+    assert e.value.code == kvm.KVM_ERANGE
+    torch.cuda.synchronize()
+    assert same_bits(k_host, canary_pool(k_host.shape))
+    kvm.swap([1], [2], False, *ptrs, slab, 256, 256, s)                   # true sizes still work afterwards
+    torch.cuda.synchronize()
+    assert same_bits(k_host[2], k_gpu[1].cpu())
