@@ -109,6 +109,33 @@ int main()
     EXPECT(kvm_copy_plain(fake_k, fake_v, -1, nullptr) == KVM_EINVAL);
     EXPECT(kvm_copy_plain(fake_k, fake_v, 0, nullptr) == KVM_OK);
 
+    EXPECT(kvm_copy_plain(fake_k, fake_v, 16, nullptr) == KVM_EINVAL);   // not device memory
+
+    // the swap plan touches no device: run lists of many shapes through it
+    int64_t sp[4];
+    EXPECT(kvm_swap_plan(ci.data(), di.data(), 1, 64, nullptr) == KVM_EINVAL);
+    EXPECT(kvm_swap_plan(nullptr, di.data(), 1, 64, sp) == KVM_EINVAL);
+    EXPECT(kvm_swap_plan(ci.data(), di.data(), 1, 0, sp) == KVM_EINVAL);
+    EXPECT(kvm_swap_plan(nullptr, nullptr, 0, 64, sp) == KVM_OK && sp[1] == 0);
+    for (int round = 0; round < 200; ++round) {
+        const int64_t n = (int64_t)(rng() % 3000);
+        std::vector<int64_t> a((size_t)n), b((size_t)n);
+        int64_t runs = n > 0 ? 1 : 0;
+        for (int64_t i = 0; i < n; ++i) {
+            const bool follow = i > 0 && rng() % 3 != 0;
+            a[(size_t)i] = follow ? a[(size_t)i - 1] + 1 : (int64_t)(rng() % 100000);
+            b[(size_t)i] = follow ? b[(size_t)i - 1] + 1 : (int64_t)(rng() % 100000);
+            if (i > 0 && !(a[(size_t)i] == a[(size_t)i - 1] + 1 && b[(size_t)i] == b[(size_t)i - 1] + 1)) ++runs;
+        }
+        const int64_t slab = (int64_t)1 << (rng() % 24);
+        EXPECT(kvm_swap_plan(a.data(), b.data(), n, slab, sp) == KVM_OK);
+        EXPECT(sp[1] == runs);
+        const int64_t want = runs > 0 && n * slab / runs < (2 << 20) ? 1 : 2;
+        EXPECT(sp[0] == want);
+        EXPECT(sp[2] == (want == 1 ? (n + 431) / 432 : 0));
+        if (failures) break;
+    }
+
     // the divider arithmetic, many operands
     for (int i = 0; i < 200000; ++i) {
         const uint32_t d = (uint32_t)(rng() >> (rng() % 40)) | 1u;
