@@ -1097,13 +1097,25 @@ int kvm_swap(const int64_t *src_ids, const int64_t *dst_ids, int64_t n, int is_s
     char *dst_k = (char *)(is_swap_in ? k_gpu : k_host), *dst_v = (char *)(is_swap_in ? v_gpu : v_host);
     hipStream_t st = (hipStream_t)stream;
 
-    const int64_t mode = swap_mode_for(pairs.data(), n, slab_bytes, nullptr);
+    int64_t mode = swap_mode_for(pairs.data(), n, slab_bytes, nullptr);
+
+    // The kernel needs the pinned pools mapped into the device's address space (the default
+    // for hipHostMalloc and for torch's pinned tensors).  When the choice was the library's
+    // own, pools that are not mapped fall back to the copy engines; a forced mode 1 reports it.
+    void *dk = nullptr, *dv = nullptr;
+    if (mode == 1) {
+        const hipError_t ek = hipHostGetDevicePointer(&dk, k_host, 0);
+        const hipError_t ev = ek == hipSuccess ? hipHostGetDevicePointer(&dv, v_host, 0) : ek;
+        if (ev != hipSuccess) {
+            (void)hipGetLastError();
+            if (opt_swap_mode.load() != 3)
+                return fail(KVM_EHIP, "host pools are not mapped for device access: %s", hipGetErrorString(ev));
+            mode = 2;
+        }
+    }
 
     if (mode == 1) {
         // One gather launch; the pinned pools are read or written in place over the host link.
-        void *dk = nullptr, *dv = nullptr;
-        KVM_HIP(hipHostGetDevicePointer(&dk, k_host, 0));
-        KVM_HIP(hipHostGetDevicePointer(&dv, v_host, 0));
         if (is_swap_in) { src_k = (char *)dk; src_v = (char *)dv; }
         else { dst_k = (char *)dk; dst_v = (char *)dv; }
         Seg s{};
