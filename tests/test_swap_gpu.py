@@ -247,3 +247,34 @@ def test_swap_pools_that_claim_more_than_their_allocation_are_refused(kvm, swap_
     kvm.swap([1], [2], False, *ptrs, slab, 256, 256, s)                   # true sizes still work afterwards
     torch.cuda.synchronize()
     assert same_bits(k_host[2], k_gpu[1].cpu())
+
+
+def test_swap_kernel_replays_inside_a_hip_graph(kvm):
+    """The copy-kernel form of the swap is one launch on the current stream, so it can be
+    captured; every replay must move what the GPU pool holds at that time."""
+    old = kvm.get_option("swap_mode")
+    kvm.set_option("swap_mode", 1)
+    try:
+        k_gpu, v_gpu, k_host, v_host = pools(10, 8, seed=21)
+        src, dst = [9, 2, 3, 4, 0], [1, 5, 6, 7, 3]
+        side = torch.cuda.Stream()
+        with torch.cuda.stream(side):                   # warm-up outside the capture
+            do_swap(kvm, src, dst, False, k_gpu, v_gpu, k_host, v_host, stream=side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            do_swap(kvm, src, dst, False, k_gpu, v_gpu, k_host, v_host)
+        for replay in range(3):
+            k_gpu.copy_(rand_pool(k_gpu.shape, 300 + replay).cuda())      # eager work between replays
+            v_gpu.copy_(rand_pool(v_gpu.shape, 400 + replay).cuda())
+            k_host.copy_(canary_pool(k_host.shape))
+            v_host.copy_(canary_pool(v_host.shape))
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            want_k, want_v = canary_pool(k_host.shape), canary_pool(v_host.shape)
+            oracle.swap_c(src, dst, k_gpu.cpu(), want_k)
+            oracle.swap_c(src, dst, v_gpu.cpu(), want_v)
+            assert same_bits(k_host, want_k) and same_bits(v_host, want_v), replay
+    finally:
+        kvm.set_option("swap_mode", old)
