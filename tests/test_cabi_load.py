@@ -136,3 +136,15 @@ def test_row_of_a_tile_is_computed_without_a_divider_exactly(kvm):
             if 0 <= n < 2**32:
                 assert kvm.lib.kvm_debug_divide(n, d) == n // d, (n, d)
     assert kvm.lib.kvm_debug_divide(5, 0) == 2**32 - 1
+
+
+def test_the_package_refuses_to_import_without_its_libraries(tmp_path):
+    """No CPU fallback: without the built HIP library the package fails at import, loudly."""
+    import subprocess
+    import sys
+
+    env = dict(os.environ, KVMOVE_LIB_DIR=str(tmp_path))
+    run = subprocess.run([sys.executable, "-c", "import distserve_amd"], capture_output=True, text=True, env=env,
+                         cwd=os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+    assert run.returncode != 0
+    assert "libkvmove.so" in run.stderr and "build" in run.stderr.lower()
