@@ -412,3 +412,60 @@ def test_ops_with_other_dtypes_block_sizes_and_head_sizes(kvm, dtype, block_size
     for u, w in enumerate(dec.workers[0]):
         assert same_bits(w.k_cache.cpu(), want_k[u]) and same_bits(w.v_cache.cpu(), want_v[u]), u
     kvm.reset()
+
+
+def test_tokens_written_by_the_producer_come_back_token_for_token(kvm):
+    """Producer-to-consumer contract at token level.  A prefill stand-in writes each token's
+    K and V vectors into the context ranks' pools the way the layout prescribes
+    (block = table[t // B], slot = t % B, rank-local layer and head); after the hand-off
+    (context TP2/PP2 -> decoding TP4), a swap-out and a swap-in, every decoding rank must
+    hold exactly those vectors at the slots its own block table names."""
+    kvm.reset()
+    L, H, D, B = 4, 8, 32, 16
+    model = ModelConfig.from_kv_shape(L, H, D)
+    cache = CacheConfig(B, 64)
+    ctx = ContextStageLLMEngine(model, ParallelConfig(2, 0, 2, 0), cache)
+    dec = DecodingStageLLMEngine(model, ParallelConfig(4, 0, 1, 0), cache,
+                                 clear_migrated_blocks_callback=ctx.clear_migrated_blocks_callback)
+    ctx._init_kvcache(16, 0)
+    dec._init_kvcache(20, 12)
+    dec.register_kvcache_mem_handles(ctx.parallel_config, ctx.kv_cache_mem_handles)
+    ctx.block_manager.allocate_blocks(create_request(20, 90))               # shift both tables
+    dec.block_manager.allocate_blocks(create_request(50, 91))
+    n_tokens = 83
+    gen = torch.Generator().manual_seed(77)
+    tok_k = (torch.rand((n_tokens, L, H, D), generator=gen) * 2 - 1).half()  # [token, layer, head, dim]
+    tok_v = (torch.rand((n_tokens, L, H, D), generator=gen) * 2 - 1).half()
+    req = create_request(n_tokens, 0)
+    ctx.block_manager.allocate_blocks(req)
+    table = ctx.block_manager.get_block_table(0)
+    for p, row in enumerate(ctx.workers):                                   # the producer
+        for t, w in enumerate(row):
+            layers, heads = slice(p * 2, p * 2 + 2), slice(t * 4, t * 4 + 4)
+            for tok in range(n_tokens):
+                w.k_cache[table[tok // B], :, :, tok % B, :] = tok_k[tok, layers, heads].cuda()
+                w.v_cache[table[tok // B], :, :, tok % B, :] = tok_v[tok, layers, heads].cuda()
+    req.add_generated_token("x", 1)
+    dec._migrate_blocks(ctx.on_prefill_finished(req))
+    assert 0 not in ctx.block_manager.block_table
+
+    def check(where):
+        table = dec.block_manager.get_block_table(0)
+        idx = torch.tensor([table[tok // B] for tok in range(n_tokens)])
+        slot = torch.tensor([tok % B for tok in range(n_tokens)])
+        for u, w in enumerate(dec.workers[0]):                              # the consumer: 2 heads per rank
+            heads = slice(u * 2, u * 2 + 2)
+            k_pool, v_pool = (w.k_cache, w.v_cache) if where == "gpu" else (w.k_swap, w.v_swap)
+            got_k = k_pool.cpu()[idx, :, :, slot, :]                        # [token, layer, head, dim]
+            got_v = v_pool.cpu()[idx, :, :, slot, :]
+            assert same_bits(got_k, tok_k[:, :, heads]) and same_bits(got_v, tok_v[:, :, heads]), (where, u)
+
+    torch.cuda.synchronize()
+    check("gpu")
+    dec.block_manager.swap_out_requests([req])
+    dec._remote_call_all_workers_async("wait_for_all_swap_out")
+    check("host")
+    dec.block_manager.swap_in_requests([req])
+    dec._remote_call_all_workers_async("wait_for_all_swap_in")
+    check("gpu")
+    kvm.reset()
