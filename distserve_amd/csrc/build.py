@@ -2,6 +2,8 @@
 
 ``libkvmove.so``        hand-written HIP kernels + the C ABI (``include/kvmove.h``); no torch.
 ``libkvmove_torch.so``  torch op shim registering ``block_migration_ops`` / ``swapping_ops``.
+``libkvmove_torch_alt.so``  the same ops as ``kvmove_block_migration_ops`` / ``kvmove_swapping_ops``,
+                        for a process that keeps another registration of DistServe's names.
 
 Run as ``python distserve_amd/csrc/build.py`` (a plain script on purpose: it must work
 when the libraries are missing or stale, so it does not import the package, which loads
@@ -22,6 +24,8 @@ INCLUDE_DIR = os.path.join(REPO_DIR, "include")
 
 KVMOVE_LIB = os.path.join(LIB_DIR, "libkvmove.so")
 TORCH_LIB = os.path.join(LIB_DIR, "libkvmove_torch.so")
+TORCH_ALT_LIB = os.path.join(LIB_DIR, "libkvmove_torch_alt.so")
+ALT_NAMESPACES = ("kvmove_block_migration_ops", "kvmove_swapping_ops")
 
 GPU_ARCH = "gfx950"
 ROCM_HOME = os.environ.get("ROCM_PATH", "/opt/rocm")
@@ -50,7 +54,7 @@ def build_kvmove() -> str:
     return KVMOVE_LIB
 
 
-def build_torch_shim() -> str:
+def build_torch_shim(alt: bool = False) -> str:
     import torch
     from torch.utils import cpp_extension
 
@@ -62,19 +66,24 @@ def build_torch_shim() -> str:
            f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}",
            f"-I{INCLUDE_DIR}", f"-I{os.path.join(ROCM_HOME, 'include')}"]
     cmd += [f"-I{p}" for p in cpp_extension.include_paths()]
-    cmd += [os.path.join(CSRC_DIR, "kvmove_torch.cpp"), "-o", TORCH_LIB,
+    out = TORCH_LIB
+    if alt:
+        out = TORCH_ALT_LIB
+        cmd += [f"-DKVM_MIGRATION_NS={ALT_NAMESPACES[0]}", f"-DKVM_SWAP_NS={ALT_NAMESPACES[1]}"]
+    cmd += [os.path.join(CSRC_DIR, "kvmove_torch.cpp"), "-o", out,
             f"-L{LIB_DIR}", "-lkvmove", "-Wl,-rpath,$ORIGIN",
             f"-L{torch_lib_dir}", "-lc10", "-lc10_hip", "-ltorch_cpu", "-ltorch", "-Wl,--no-as-needed"]
     _run(cmd)
-    return TORCH_LIB
+    return out
 
 
 def build_all() -> None:
     build_kvmove()
     build_torch_shim()
+    build_torch_shim(alt=True)
 
 
 if __name__ == "__main__":
     build_all()
-    print("built:", KVMOVE_LIB, TORCH_LIB)
+    print("built:", KVMOVE_LIB, TORCH_LIB, TORCH_ALT_LIB)
     sys.exit(0)

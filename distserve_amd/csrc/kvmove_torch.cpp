@@ -123,7 +123,19 @@ void swap(std::vector<int64_t> source_block_ids, std::vector<int64_t> target_blo
 
 }  // namespace
 
-TORCH_LIBRARY(block_migration_ops, m)
+// The op namespaces are DistServe's.  A process that must also keep another library's
+// registration of the same names (two definitions of one op are an error in torch) loads
+// the build of this file with -DKVM_MIGRATION_NS=... -DKVM_SWAP_NS=... instead, and calls
+// the ops under those names.
+#ifndef KVM_MIGRATION_NS
+#define KVM_MIGRATION_NS block_migration_ops
+#endif
+#ifndef KVM_SWAP_NS
+#define KVM_SWAP_NS swapping_ops
+#endif
+#define KVM_TORCH_LIBRARY(ns, m) TORCH_LIBRARY(ns, m)
+
+KVM_TORCH_LIBRARY(KVM_MIGRATION_NS, m)
 {
     m.def("get_ipc_mem_handle(Tensor t) -> int[]", get_ipc_mem_handle);
     m.def("register_ipc_mem_handle(int[] k_handle, int[] v_handle, int num_layers, int num_heads, "
@@ -135,7 +147,7 @@ TORCH_LIBRARY(block_migration_ops, m)
           migrate_blocks);
 }
 
-TORCH_LIBRARY(swapping_ops, m)
+KVM_TORCH_LIBRARY(KVM_SWAP_NS, m)
 {
     m.def("swap(int[] source_block_ids, int[] target_block_ids, bool is_swap_in, Tensor k_cache, "
           "Tensor v_cache, Tensor k_swap, Tensor v_swap) -> ()",

@@ -148,3 +148,21 @@ def test_the_package_refuses_to_import_without_its_libraries(tmp_path):
                          cwd=os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
     assert run.returncode != 0
     assert "libkvmove.so" in run.stderr and "build" in run.stderr.lower()
+
+
+def test_the_alternate_namespace_build_registers_the_same_schemas_beside_the_first():
+    """A process that keeps another library's block_migration_ops / swapping_ops loads the
+    second build of the shim; both can live in one process."""
+    import torch
+
+    import distserve_amd
+
+    torch.ops.load_library(os.path.join(os.path.dirname(distserve_amd.TORCH_LIB_PATH), "libkvmove_torch_alt.so"))
+
+    def args_of(op):
+        return str(op.default._schema).split("(", 1)[1]
+
+    for name in ("get_ipc_mem_handle", "register_ipc_mem_handle", "migrate_blocks"):
+        assert args_of(getattr(torch.ops.kvmove_block_migration_ops, name)) == \
+            args_of(getattr(torch.ops.block_migration_ops, name))
+    assert args_of(torch.ops.kvmove_swapping_ops.swap) == args_of(torch.ops.swapping_ops.swap)
