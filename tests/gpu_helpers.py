@@ -32,12 +32,35 @@ def upload_and_register(g: oracle.Geom, src_k: List[List[torch.Tensor]], src_v: 
     return dev_k, dev_v
 
 
+GUARD = 4096   # elements of canary kept on either side of a destination pool
+
+
+def guarded_canary_pool(shape, dtype=torch.float16):
+    """A canary-filled GPU pool that sits in the middle of a larger canary-filled buffer;
+    returns (pool view, whole buffer).  The margins must still hold the canary afterwards:
+    a write that strays past either end of the pool lands there."""
+    n = 1
+    for d in shape:
+        n *= d
+    whole = canary_pool((n + 2 * GUARD,), dtype).cuda()
+    return whole[GUARD:GUARD + n].view(shape), whole
+
+
+def guards_intact(whole: torch.Tensor) -> bool:
+    margin = canary_pool((GUARD,), whole.dtype)
+    got = whole.cpu()
+    return (torch.equal(got[:GUARD].view(torch.uint8), margin.view(torch.uint8))
+            and torch.equal(got[-GUARD:].view(torch.uint8), margin.view(torch.uint8)))
+
+
 def gpu_migrate(g: oracle.Geom, ci, di, nb_dst: int, dtype=torch.float16):
-    """Runs kvm_migrate into canary-filled destination pools; returns them on the CPU."""
-    dst_k = canary_pool(g.dec_pool_shape(nb_dst), dtype).cuda()
-    dst_v = canary_pool(g.dec_pool_shape(nb_dst), dtype).cuda()
+    """Runs kvm_migrate into canary-filled destination pools; returns them on the CPU.  The
+    pools have canary margins on both sides, which must survive."""
+    dst_k, whole_k = guarded_canary_pool(g.dec_pool_shape(nb_dst), dtype)
+    dst_v, whole_v = guarded_canary_pool(g.dec_pool_shape(nb_dst), dtype)
     cabi.migrate(kvm_geom(g), ci, di, dst_k.data_ptr(), dst_v.data_ptr(), nb_dst, stream_handle())
     torch.cuda.synchronize()
+    assert guards_intact(whole_k) and guards_intact(whole_v), "a write strayed outside the destination pool"
     return dst_k.cpu(), dst_v.cpu()
 
 

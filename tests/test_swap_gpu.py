@@ -6,7 +6,7 @@ import torch
 
 import oracle
 from distserve_amd import workloads
-from gpu_helpers import kvm_geom, upload_and_register
+from gpu_helpers import GUARD, kvm_geom, upload_and_register
 from helpers import canary_pool, geom_of, make_src_pools, rand_pool, same_bits
 
 pytestmark = pytest.mark.gpu
@@ -28,6 +28,29 @@ def pools(n_gpu, n_host, seed, block=BLOCK):
     k_host = canary_pool((n_host,) + block).pin_memory()
     v_host = canary_pool((n_host,) + block).pin_memory()
     return k_gpu, v_gpu, k_host, v_host
+
+
+def guarded_pools(n_gpu, n_host, seed, block):
+    """Like pools(), with canary margins on both sides of every pool; also returns a check
+    that the margins still hold the canary (no write strayed past a pool's ends)."""
+    def inside(whole, n):
+        return whole[GUARD:GUARD + n * whole_block].view((n,) + block)
+
+    whole_block = 1
+    for d in block:
+        whole_block *= d
+    wholes = [canary_pool((n_gpu * whole_block + 2 * GUARD,)).cuda() for _ in range(2)]
+    wholes += [canary_pool((n_host * whole_block + 2 * GUARD,)).pin_memory() for _ in range(2)]
+    k_gpu, v_gpu = inside(wholes[0], n_gpu), inside(wholes[1], n_gpu)
+    k_gpu.copy_(rand_pool((n_gpu,) + block, seed))
+    v_gpu.copy_(rand_pool((n_gpu,) + block, seed + 1))
+    k_host, v_host = inside(wholes[2], n_host), inside(wholes[3], n_host)
+    margin = canary_pool((GUARD,))
+
+    def margins_intact():
+        return all(same_bits(w[:GUARD].cpu(), margin) and same_bits(w[-GUARD:].cpu(), margin) for w in wholes)
+
+    return k_gpu, v_gpu, k_host, v_host, margins_intact
 
 
 def do_swap(kvm, src, dst, swap_in, k_gpu, v_gpu, k_host, v_host, stream=None):
@@ -210,7 +233,7 @@ def test_random_slab_sizes_lists_and_pool_sizes(kvm, swap_mode):
     for case in range(60):
         block = (rng.choice([1, 2, 5]), rng.choice([1, 3, 4]), rng.choice([1, 2, 16]), rng.choice([1, 3, 8, 40, 128]))
         n_gpu, n_host = rng.randint(2, 14), rng.randint(1, 14)
-        k_gpu, v_gpu, k_host, v_host = pools(n_gpu, n_host, seed=100 + case, block=block)
+        k_gpu, v_gpu, k_host, v_host, margins_intact = guarded_pools(n_gpu, n_host, 100 + case, block)
         k0, v0 = k_gpu.cpu(), v_gpu.cpu()
         n = rng.randint(0, min(n_gpu, n_host))
         if rng.random() < 0.5:                       # a run of consecutive blocks on both sides
@@ -231,6 +254,7 @@ def test_random_slab_sizes_lists_and_pool_sizes(kvm, swap_mode):
         oracle.swap_c(out_dst, in_dst, want_k, exp_k)
         oracle.swap_c(out_dst, in_dst, want_v, exp_v)
         assert same_bits(k_gpu.cpu(), exp_k) and same_bits(v_gpu.cpu(), exp_v), (case, block, out_dst, in_dst)
+        assert margins_intact(), (case, block)
 
 
 def test_swap_pools_that_claim_more_than_their_allocation_are_refused(kvm, swap_mode):
