@@ -23,7 +23,9 @@ def run_bench(*flags, timeout=300):
     gc.collect()
     torch.cuda.synchronize()
     torch.cuda.empty_cache()
-    torch._C._host_emptyCache()
+    release_pinned = getattr(torch._C, "_host_emptyCache", None)
+    if release_pinned is not None:
+        release_pinned()
     out = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), *flags], cwd=ROOT,
                          capture_output=True, text=True, timeout=timeout)
     if out.returncode != 0:
