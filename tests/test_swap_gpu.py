@@ -302,3 +302,70 @@ def test_swap_kernel_replays_inside_a_hip_graph(kvm):
             assert same_bits(k_host, want_k) and same_bits(v_host, want_v), replay
     finally:
         kvm.set_option("swap_mode", old)
+
+
+def test_swaps_and_a_migration_from_several_host_threads(kvm, swap_mode):
+    """The library may be entered concurrently: two threads swap their own pools out and
+    back on their own streams while a third migrates, each result checked on its own."""
+    import threading
+
+    kvm.reset()
+    g = oracle.Geom(2, 4, 16, 64, 2)
+    nb = 48
+    src_k, src_v = make_src_pools(g, nb, 61), make_src_pools(g, nb, 62)
+    keep = upload_and_register(g, src_k, src_v)
+    errors, results = [], {}
+
+    def swapper(tid):
+        try:
+            torch.cuda.set_device(0)
+            stream = torch.cuda.Stream()
+            rng = torch.Generator().manual_seed(200 + tid)
+            k_gpu, v_gpu, k_host, v_host = pools(24, 20, seed=70 + tid)
+            want_gk, want_gv = k_gpu.cpu(), v_gpu.cpu()
+            want_hk, want_hv = canary_pool(k_host.shape), canary_pool(v_host.shape)
+            for _ in range(12):
+                n = int(torch.randint(1, 9, (1,), generator=rng))
+                a = torch.randperm(24, generator=rng)[:n].tolist()
+                b = torch.randperm(20, generator=rng)[:n].tolist()
+                c = torch.randperm(24, generator=rng)[:n].tolist()
+                do_swap(kvm, a, b, False, k_gpu, v_gpu, k_host, v_host, stream=stream)
+                do_swap(kvm, b, c, True, k_gpu, v_gpu, k_host, v_host, stream=stream)
+                oracle.swap_c(a, b, want_gk, want_hk)
+                oracle.swap_c(a, b, want_gv, want_hv)
+                oracle.swap_c(b, c, want_hk, want_gk)
+                oracle.swap_c(b, c, want_hv, want_gv)
+            stream.synchronize()
+            results[tid] = (same_bits(k_gpu.cpu(), want_gk) and same_bits(v_gpu.cpu(), want_gv)
+                            and same_bits(k_host, want_hk) and same_bits(v_host, want_hv))
+        except Exception as e:      # noqa: BLE001
+            errors.append((tid, repr(e)))
+
+    def migrator():
+        try:
+            torch.cuda.set_device(0)
+            stream = torch.cuda.Stream()
+            rng = torch.Generator().manual_seed(300)
+            dk, dv = canary_pool(g.dec_pool_shape(nb)).cuda(), canary_pool(g.dec_pool_shape(nb)).cuda()
+            want_k, want_v = canary_pool(g.dec_pool_shape(nb)), canary_pool(g.dec_pool_shape(nb))
+            for _ in range(30):
+                n = int(torch.randint(1, 9, (1,), generator=rng))
+                ci = torch.randint(0, nb, (n,), generator=rng).tolist()
+                di = torch.randperm(nb, generator=rng)[:n].tolist()
+                kvm.migrate(kvm_geom(g), ci, di, dk.data_ptr(), dv.data_ptr(), nb, stream.cuda_stream)
+                oracle.migrate_c(g, src_k, ci, di, want_k)
+                oracle.migrate_c(g, src_v, ci, di, want_v)
+            stream.synchronize()
+            results["migrate"] = same_bits(dk.cpu(), want_k) and same_bits(dv.cpu(), want_v)
+        except Exception as e:      # noqa: BLE001
+            errors.append(("migrate", repr(e)))
+
+    threads = [threading.Thread(target=swapper, args=(t,)) for t in range(2)] + [threading.Thread(target=migrator)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    assert results == {0: True, 1: True, "migrate": True}, results
+    del keep
+    kvm.reset()
