@@ -849,14 +849,16 @@ int checked_pool(const void *p, uint64_t need, bool on_device, const char *what)
 struct Fork {
     hipStream_t side = nullptr;
     hipEvent_t forked = nullptr, joined = nullptr;
+    std::mutex in_use;   // held while one call forks, enqueues and joins: the events are per set
 };
-std::mutex g_fork_mu;
+std::mutex g_fork_mu;    // guards the map only (std::map keeps its nodes where they are)
 std::map<std::pair<int, bool>, Fork> g_forks;
 
 int get_fork(bool is_swap_in, Fork **out)
 {
     int dev = 0;
     KVM_HIP(hipGetDevice(&dev));
+    std::lock_guard<std::mutex> lock(g_fork_mu);
     Fork &f = g_forks[{dev, is_swap_in}];
     if (!f.side) {
         KVM_HIP(hipStreamCreateWithFlags(&f.side, hipStreamNonBlocking));
@@ -1138,8 +1140,8 @@ int kvm_swap(const int64_t *src_ids, const int64_t *dst_ids, int64_t n, int is_s
     Fork *fork = nullptr;
     std::unique_lock<std::mutex> fork_lock;
     if (mode == 2) {
-        fork_lock = std::unique_lock<std::mutex>(g_fork_mu);
         if (int rc = get_fork(is_swap_in != 0, &fork)) return rc;
+        fork_lock = std::unique_lock<std::mutex>(fork->in_use);
         KVM_HIP(hipEventRecord(fork->forked, st));
         KVM_HIP(hipStreamWaitEvent(fork->side, fork->forked, 0));
         st_v = fork->side;
