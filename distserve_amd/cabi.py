@@ -18,12 +18,13 @@ KVM_ENOTREG = -4
 KVM_EHIP = -5
 KVM_EHANDLE = -6
 KVM_EMISMATCH = -7
-KVM_HANDLE_WORDS = 8
+KVM_HANDLE_WORDS = 17
+KVM_IPC_MAX_ALLOC_BYTES = 1 << 31
 
 # every symbol include/kvmove.h declares
 EXPORTS = (
     "kvm_version", "kvm_last_error", "kvm_get_mem_handle", "kvm_register_mem_handle",
-    "kvm_register_source", "kvm_reset", "kvm_migrate", "kvm_swap", "kvm_copy_plain",
+    "kvm_register_source", "kvm_reset", "kvm_opened_handles", "kvm_migrate", "kvm_swap", "kvm_copy_plain",
     "kvm_set_option", "kvm_get_option", "kvm_migrate_plan", "kvm_swap_plan", "kvm_debug_divide",
 )
 
@@ -41,6 +42,7 @@ class KvmGeom(ctypes.Structure):
         ("ctx_pp_size", ctypes.c_int32), ("ctx_tp_size", ctypes.c_int32),
         ("dec_pp_size", ctypes.c_int32), ("dec_tp_size", ctypes.c_int32),
         ("dec_pp_rank", ctypes.c_int32), ("dec_tp_rank", ctypes.c_int32),
+        ("ctx_instance", ctypes.c_int64),
     ]
 
 
@@ -58,9 +60,11 @@ def _load() -> ctypes.CDLL:
     lib.kvm_version.restype = ctypes.c_int
     lib.kvm_last_error.restype = ctypes.c_char_p
     lib.kvm_get_mem_handle.argtypes = [vp, i64, ip]
-    lib.kvm_register_mem_handle.argtypes = [ip, ip, i64, i64, ip, ip]
-    lib.kvm_register_source.argtypes = [i32, i32, i32, i32, i64, i64, vp, vp, i64]
+    lib.kvm_register_mem_handle.argtypes = [ip, ip, i64, i64, ip, ip, i64]
+    lib.kvm_register_source.argtypes = [i32, i32, i32, i32, i64, i64, vp, vp, i64, i64]
     lib.kvm_reset.argtypes = []
+    lib.kvm_opened_handles.argtypes = []
+    lib.kvm_opened_handles.restype = i64
     lib.kvm_migrate.argtypes = [ctypes.POINTER(KvmGeom), ip, ip, i64, vp, vp, i64, vp]
     lib.kvm_swap.argtypes = [ip, ip, i64, ctypes.c_int, vp, vp, vp, vp, i64, i64, i64, vp]
     lib.kvm_copy_plain.argtypes = [vp, vp, i64, vp]
@@ -73,7 +77,8 @@ def _load() -> ctypes.CDLL:
     lib.kvm_debug_divide.restype = ctypes.c_uint32
     for name in EXPORTS:
         fn = getattr(lib, name)
-        if name not in ("kvm_last_error", "kvm_get_option", "kvm_version", "kvm_debug_divide"):
+        if name not in ("kvm_last_error", "kvm_get_option", "kvm_version", "kvm_debug_divide",
+                        "kvm_opened_handles"):
             fn.restype = ctypes.c_int
     return lib
 
@@ -102,9 +107,9 @@ def version() -> int:
 
 
 def geom(num_layers, num_kv_heads, block_size, head_dim, dtype_bytes, ctx_pp=1, ctx_tp=1,
-         dec_pp=1, dec_tp=1, dec_pp_rank=0, dec_tp_rank=0) -> KvmGeom:
+         dec_pp=1, dec_tp=1, dec_pp_rank=0, dec_tp_rank=0, ctx_instance=0) -> KvmGeom:
     return KvmGeom(num_layers, num_kv_heads, block_size, head_dim, dtype_bytes,
-                   ctx_pp, ctx_tp, dec_pp, dec_tp, dec_pp_rank, dec_tp_rank)
+                   ctx_pp, ctx_tp, dec_pp, dec_tp, dec_pp_rank, dec_tp_rank, ctx_instance)
 
 
 def get_mem_handle(dev_ptr: int, nbytes: int) -> List[int]:
@@ -113,23 +118,29 @@ def get_mem_handle(dev_ptr: int, nbytes: int) -> List[int]:
     return list(out)
 
 
-def register_mem_handle(k_handle, v_handle, num_layers, num_kv_heads, context_pc, decoding_pc) -> None:
+def register_mem_handle(k_handle, v_handle, num_layers, num_kv_heads, context_pc, decoding_pc,
+                        ctx_instance: int = 0) -> None:
     if len(k_handle) != KVM_HANDLE_WORDS or len(v_handle) != KVM_HANDLE_WORDS:
         raise KvmError(KVM_EHANDLE, f"a memory handle has {KVM_HANDLE_WORDS} words")
     if len(context_pc) != 4 or len(decoding_pc) != 4:
         raise KvmError(KVM_EINVAL, "parallel configs are [tp_size, tp_rank, pp_size, pp_rank]")
     _check(lib.kvm_register_mem_handle(_arr(k_handle), _arr(v_handle), num_layers, num_kv_heads,
-                                       _arr(context_pc), _arr(decoding_pc)))
+                                       _arr(context_pc), _arr(decoding_pc), ctx_instance))
 
 
 def register_source(ctx_pp_size, ctx_tp_size, pp_rank, tp_rank, num_layers, num_kv_heads,
-                    k_ptr: int, v_ptr: int, nbytes_each: int) -> None:
+                    k_ptr: int, v_ptr: int, nbytes_each: int, ctx_instance: int = 0) -> None:
     _check(lib.kvm_register_source(ctx_pp_size, ctx_tp_size, pp_rank, tp_rank, num_layers, num_kv_heads,
-                                   k_ptr, v_ptr, nbytes_each))
+                                   k_ptr, v_ptr, nbytes_each, ctx_instance))
 
 
 def reset() -> None:
     _check(lib.kvm_reset())
+
+
+def opened_handles() -> int:
+    """Allocations of other processes that registration currently keeps mapped."""
+    return lib.kvm_opened_handles()
 
 
 def migrate(g: KvmGeom, ctx_idx: Sequence[int], dec_idx: Sequence[int], dst_k: int, dst_v: int,
@@ -177,5 +188,5 @@ def migrate_plan(g: KvmGeom, n: int, dst_k: int, dst_v: int) -> dict:
     out = (ctypes.c_int64 * 8)()
     _check(lib.kvm_migrate_plan(ctypes.byref(g), n, dst_k, dst_v, out))
     keys = ("workgroups_per_block", "threads", "vector_bytes", "segments", "launches", "payload_bytes_per_block",
-            "simple_kernel")
+            "simple_kernel", "max_work_items")
     return dict(zip(keys, list(out)))

@@ -404,19 +404,47 @@ std::atomic<int64_t> *find_opt(const char *name)
     return nullptr;
 }
 
-// ---- registry of context pools, keyed by (pp_rank, tp_rank)
+// ---- registry of context pools, keyed by (context instance, pp_rank, tp_rank)
 
 struct Source {
     int32_t ctx_pp_size, ctx_tp_size;
     int64_t num_layers, num_kv_heads;
     const char *k, *v;
     int64_t nbytes;
+    const char *map_k, *map_v;   // local base of the other process's allocation each pool lies in, or null
 };
 
-std::mutex g_mu;
-std::map<std::pair<int32_t, int32_t>, Source> g_sources;
+using SourceKey = std::tuple<int64_t, int32_t, int32_t>;
 
-constexpr int64_t kHandleMagic = 0x4b564d4f56453031LL;  // "KVMOVE01"
+std::mutex g_mu;
+std::map<SourceKey, Source> g_sources;
+
+// Allocations of other processes that registration has mapped into this one.  One entry per
+// (exporting process, allocation): hipIpcOpenMemHandle is called once however many pools lie
+// in the allocation, and the mapping stays until kvm_reset.
+struct Opened {
+    int64_t pid, remote_base, size;
+    hipIpcMemHandle_t handle;
+    char *local_base;
+};
+std::vector<Opened> g_opened;   // guarded by g_mu
+
+// Handle words (int64 each).
+enum {
+    kHwMagic = 0, kHwPid, kHwDevice, kHwPtr, kHwBytes, kHwAllocBase, kHwAllocSize, kHwFlags,
+    kHwIpc = 8,                                  // 8 words = the 64 bytes of a hipIpcMemHandle_t
+    kHwCheck = 16,
+};
+static_assert(sizeof(hipIpcMemHandle_t) == 64 && kHwCheck + 1 == KVM_HANDLE_WORDS, "handle layout");
+constexpr int64_t kHandleMagic = 0x4b564d4f56453032LL;  // "KVMOVE02"
+constexpr int64_t kHandleHasIpc = 1;                    // flag: words 8..15 hold an exported IPC handle
+
+int64_t handle_check(const int64_t *h)
+{
+    uint64_t x = 0x5a5a5a5a5a5a5a5aull;
+    for (int i = 0; i < kHwCheck; ++i) x = ((x << 7) | (x >> 57)) ^ (uint64_t)h[i];
+    return (int64_t)x;
+}
 
 // ---- kernel table
 
@@ -567,7 +595,9 @@ int check_geom(const KvmGeom *g)
     return KVM_OK;
 }
 
-int build_plan(const KvmGeom *g, const void *dst_k, const void *dst_v, Plan *plan)
+// `arithmetic_only`: context ranks that are not registered count as 16-byte aligned pools of
+// unknown size at address 0, so that the launch shape can be computed without a device.
+int build_plan(const KvmGeom *g, const void *dst_k, const void *dst_v, Plan *plan, bool arithmetic_only = false)
 {
     if (int rc = check_geom(g)) return rc;
     const int64_t Lc = g->num_layers / g->ctx_pp_size, Hc = g->num_kv_heads / g->ctx_tp_size;
@@ -589,11 +619,13 @@ int build_plan(const KvmGeom *g, const void *dst_k, const void *dst_v, Plan *pla
     std::lock_guard<std::mutex> lock(g_mu);
     for (int64_t p = l0 / Lc; p * Lc < l1; ++p) {
         for (int64_t t = h0 / Hc; t * Hc < h1; ++t) {
-            auto it = g_sources.find({(int32_t)p, (int32_t)t});
-            if (it == g_sources.end())
-                return fail(KVM_ENOTREG, "context rank (pp %lld, tp %lld) is not registered",
-                            (long long)p, (long long)t);
-            const Source &src = it->second;
+            auto it = g_sources.find(SourceKey{g->ctx_instance, (int32_t)p, (int32_t)t});
+            if (it == g_sources.end() && !arithmetic_only)
+                return fail(KVM_ENOTREG, "context rank (pp %lld, tp %lld) of context instance %lld is not registered",
+                            (long long)p, (long long)t, (long long)g->ctx_instance);
+            const Source unknown{g->ctx_pp_size, g->ctx_tp_size, g->num_layers, g->num_kv_heads, nullptr, nullptr,
+                                 (int64_t)INT32_MAX * src_block, nullptr, nullptr};
+            const Source &src = it == g_sources.end() ? unknown : it->second;
             if (src.ctx_pp_size != g->ctx_pp_size || src.ctx_tp_size != g->ctx_tp_size ||
                 src.num_layers != g->num_layers || src.num_kv_heads != g->num_kv_heads)
                 return fail(KVM_EMISMATCH,
@@ -664,71 +696,114 @@ WalkFn pick_walk(int vec)
                      : kvm_walk_kernel<uint8_t>;
 }
 
+// Everything launch_copy decides about one group of up to 8 segments before it launches.
+struct Group {
+    MigrateArgs args;        // filled up to the index pairs
+    uint32_t tiles = 0;      // tiles per block of one pool kind
+    int64_t per_launch = 0;  // index pairs per launch
+    bool simple = false;
+};
+
+// A launch is a 1-D grid of 2 * work_padded workgroups of `threads` lanes, and the runtime
+// refuses a grid of 2^32 work-items or more.  plan_work pads the work of a launch by fewer
+// than 8 tiles, or not at all, so this many index pairs per launch stay below that.
+int64_t pairs_per_launch(uint32_t tiles, int threads)
+{
+    const int64_t max_tiles = (int64_t)(UINT32_MAX / (2u * (uint32_t)threads)) - 8;
+    return std::min<int64_t>(kMaxIdx, max_tiles / (int64_t)tiles);
+}
+
 // Enqueues the copy over `segs` x `pairs`, as many launches as the 4 KiB argument needs
-// (8 segments and 432 index pairs each).  `pairs == nullptr` only counts what would be
-// launched.  walk_wgs > 0 selects the link-bound form with that many workgroups per pool kind.
+// (8 segments and 432 index pairs each) and the grid limit allows.  Every launch of the call
+// is sized and checked before the first one is enqueued, so a call that cannot be launched
+// has touched nothing.  `pairs == nullptr` only counts what would be launched.  walk_wgs > 0
+// selects the link-bound form with that many workgroups per pool kind.
 int launch_copy(std::vector<Seg> segs, const IdxPair *pairs, int64_t n, char *dst_k, char *dst_v,
                 uint64_t dst_block_stride, int vec, hipStream_t stream, int64_t *out_launches,
-                int64_t *out_wgs_per_block, int *out_threads, int walk_wgs = 0, bool *out_simple = nullptr)
+                int64_t *out_wgs_per_block, int *out_threads, int walk_wgs = 0, bool *out_simple = nullptr,
+                int64_t *out_max_items = nullptr)
 {
     Launch k;
     if (int rc = pick_kernel(vec, &k)) return rc;
     // tile_bytes 0 = one shot: exactly what the workgroup's lanes hold in flight
     uint32_t tile_bytes = (uint32_t)opt_tile_bytes.load();
     if (tile_bytes == 0) tile_bytes = (uint32_t)((walk_wgs > 0 ? 256 * 4 : k.threads * k.unroll) * vec);
-    int64_t launches = 0, wgs_per_block = 0;
+    int64_t launches = 0, wgs_per_block = 0, max_items = 0;
     bool all_simple = true;
-    for (size_t s0 = 0; s0 < segs.size(); s0 += kMaxSegs) {
-        MigrateArgs args;
+    std::vector<Group> groups((segs.size() + kMaxSegs - 1) / kMaxSegs);
+    for (size_t gi = 0; gi < groups.size(); ++gi) {
+        const size_t s0 = gi * kMaxSegs;
+        Group &grp = groups[gi];
+        MigrateArgs &args = grp.args;
         args.dst_k = dst_k;
         args.dst_v = dst_v;
         args.dst_block_stride = dst_block_stride;
         args.nseg = (uint32_t)std::min<size_t>(kMaxSegs, segs.size() - s0);
-        uint32_t tiles_total = 0;
+        uint64_t tiles_total = 0;
         for (uint32_t j = 0; j < args.nseg; ++j) {
             Seg s = segs[s0 + j];
             uint32_t tiles = 0;
             tile_segment(s, tile_bytes, &tiles);
             tiles_total += tiles;
-            args.tile_end[j] = tiles_total;
+            args.tile_end[j] = (uint32_t)std::min<uint64_t>(tiles_total, UINT32_MAX);
             args.seg[j] = s;
         }
         for (uint32_t j = args.nseg; j < kMaxSegs; ++j) args.tile_end[j] = UINT32_MAX;
         args.tile_end[args.nseg - 1] = UINT32_MAX;   // nothing lies past the last segment
         // one collapsed segment of full one-shot tiles takes the short-prologue kernel
         const Seg &first = args.seg[0];
-        const bool simple = walk_wgs == 0 && k.simple_fn && opt_simple.load() && args.nseg == 1 &&
-                            first.n_rows == 1 && first.rows_per_tile == 1 && first.run_bytes % tile_bytes == 0 &&
-                            tile_bytes == (uint32_t)(k.threads * k.unroll * vec);
-        all_simple = all_simple && simple;
+        grp.simple = walk_wgs == 0 && k.simple_fn && opt_simple.load() && args.nseg == 1 &&
+                     first.n_rows == 1 && first.rows_per_tile == 1 && first.run_bytes % tile_bytes == 0 &&
+                     tile_bytes == (uint32_t)(k.threads * k.unroll * vec);
+        all_simple = all_simple && grp.simple;
         wgs_per_block += 2 * (int64_t)tiles_total;
-        // a launch is a 1-D grid of 2 * tiles * blocks workgroups, which must stay below 2^31
         if (tiles_total == 0 || tiles_total > (1u << 29))
-            return fail(KVM_EINVAL, "%u tiles per block cannot be launched", tiles_total);
-        const int64_t per_launch = std::min<int64_t>(kMaxIdx, (int64_t)((1u << 29) / tiles_total));
-        for (int64_t i0 = 0; i0 < n; i0 += per_launch) {
-            args.nidx = (uint32_t)std::min<int64_t>(per_launch, n - i0);
-            if (pairs) {
+            return fail(KVM_EINVAL, "%llu tiles per block cannot be launched", (unsigned long long)tiles_total);
+        grp.tiles = (uint32_t)tiles_total;
+        // the walking form's grid is a few workgroups whatever the work
+        grp.per_launch = walk_wgs > 0 ? std::min<int64_t>(kMaxIdx, (int64_t)(UINT32_MAX / grp.tiles))
+                                      : pairs_per_launch(grp.tiles, k.threads);
+        if (grp.per_launch < 1)
+            return fail(KVM_EINVAL, "one block is %u tiles of %d lanes per pool kind: no launch can hold it",
+                        grp.tiles, k.threads);
+        const int64_t largest = std::min<int64_t>(grp.per_launch, std::max<int64_t>(n, 1));
+        if (walk_wgs > 0) {
+            max_items = std::max<int64_t>(max_items, 2 * 256 * (int64_t)walk_wgs);
+        } else {
+            MigrateArgs probe = args;
+            probe.nidx = (uint32_t)largest;
+            plan_work(probe, grp.tiles, tile_bytes);
+            const int64_t items = 2 * (int64_t)probe.work_padded * k.threads;
+            if (items > (int64_t)UINT32_MAX)
+                return fail(KVM_EINVAL, "a launch of %lld work-items cannot be made", (long long)items);
+            max_items = std::max(max_items, items);
+        }
+        launches += n == 0 ? 1 : (n + grp.per_launch - 1) / grp.per_launch;
+    }
+    if (pairs) {
+        for (Group &grp : groups) {
+            MigrateArgs &args = grp.args;
+            for (int64_t i0 = 0; i0 < n; i0 += grp.per_launch) {
+                args.nidx = (uint32_t)std::min<int64_t>(grp.per_launch, n - i0);
                 memcpy(args.idx, pairs + i0, args.nidx * sizeof(IdxPair));
                 if (walk_wgs > 0) {
-                    const uint32_t work = tiles_total * args.nidx;
+                    const uint32_t work = grp.tiles * args.nidx;
                     hipLaunchKernelGGL(pick_walk(vec), dim3(std::min<uint32_t>((uint32_t)walk_wgs, work), 2),
-                                       dim3(256), 0, stream, args, tiles_total);
+                                       dim3(256), 0, stream, args, grp.tiles);
                 } else {
-                    plan_work(args, tiles_total, tile_bytes);
-                    hipLaunchKernelGGL(simple ? k.simple_fn : k.fn, dim3(2 * args.work_padded), dim3(k.threads),
+                    plan_work(args, grp.tiles, tile_bytes);
+                    hipLaunchKernelGGL(grp.simple ? k.simple_fn : k.fn, dim3(2 * args.work_padded), dim3(k.threads),
                                        (size_t)opt_lds_pad.load(), stream, args);
                 }
                 KVM_HIP(hipGetLastError());
             }
-            ++launches;
         }
-        if (n == 0) ++launches;
     }
     if (out_launches) *out_launches = launches;
     if (out_wgs_per_block) *out_wgs_per_block = wgs_per_block;
     if (out_threads) *out_threads = k.threads;
     if (out_simple) *out_simple = all_simple && !segs.empty();
+    if (out_max_items) *out_max_items = max_items;
     return KVM_OK;
 }
 
@@ -808,38 +883,18 @@ int check_extent(const void *p, uint64_t need, uint64_t extent, const char *what
     return KVM_OK;
 }
 
-// Pointers already checked by device_of / host_pinned (the queries cost microseconds).  Pools
-// are borrowed for as long as the caller uses them, so a base address keeps its kind and its
-// extent; a size that does not fit the remembered extent is looked up afresh before it is
-// refused (the address may belong to a newer allocation), and kvm_reset() forgets everything.
-struct Known {
-    int device;        // -1 for pinned host memory
-    uint64_t extent;   // see extent_of
-};
-std::mutex g_checked_mu;
-std::map<const void *, Known> g_checked;
-
+// A pool argument is looked up afresh on every call: the two runtime queries cost well under a
+// microsecond each, and an address remembered from an earlier call may by now belong to another,
+// smaller allocation.
 int checked_pool(const void *p, uint64_t need, bool on_device, const char *what)
 {
-    {
-        std::lock_guard<std::mutex> lock(g_checked_mu);
-        auto it = g_checked.find(p);
-        if (it != g_checked.end() && (it->second.device >= 0) == on_device &&
-            (it->second.extent == 0 || need <= it->second.extent))
-            return KVM_OK;
-    }
     int dev = -1;
     if (on_device) {
         if (int rc = device_of(p, what, &dev)) return rc;
     } else {
         if (int rc = host_pinned(p, what)) return rc;
     }
-    const uint64_t extent = extent_of(p);
-    if (int rc = check_extent(p, need, extent, what)) return rc;
-    std::lock_guard<std::mutex> lock(g_checked_mu);
-    if (g_checked.size() > 64) g_checked.clear();
-    g_checked[p] = Known{dev, extent};
-    return KVM_OK;
+    return check_extent(p, need, extent_of(p), what);
 }
 
 // A second stream (default priority) and the two events that fork it from and join it back
@@ -926,33 +981,105 @@ int kvm_get_mem_handle(const void *dev_ptr, int64_t nbytes, int64_t *out_handle)
         return fail(KVM_EINVAL, "kvm_get_mem_handle: null pointer or non-positive size");
     int dev = 0;
     if (int rc = device_of(dev_ptr, "pool", &dev)) return rc;
-    memset(out_handle, 0, sizeof(int64_t) * KVM_HANDLE_WORDS);
-    out_handle[0] = kHandleMagic;
-    out_handle[1] = (int64_t)getpid();
-    out_handle[2] = dev;
-    out_handle[3] = (int64_t)(uintptr_t)dev_ptr;
-    out_handle[4] = nbytes;
-    out_handle[5] = out_handle[0] ^ out_handle[1] ^ out_handle[2] ^ out_handle[3] ^ out_handle[4];
+    int64_t *h = out_handle;
+    memset(h, 0, sizeof(int64_t) * KVM_HANDLE_WORDS);
+    h[kHwMagic] = kHandleMagic;
+    h[kHwPid] = (int64_t)getpid();
+    h[kHwDevice] = dev;
+    h[kHwPtr] = (int64_t)(uintptr_t)dev_ptr;
+    h[kHwBytes] = nbytes;
+    // The IPC handle names a whole allocation, so the pool travels as (allocation, offset).
+    hipDeviceptr_t base = nullptr;
+    size_t size = 0;
+    if (hipMemGetAddressRange(&base, &size, (hipDeviceptr_t)dev_ptr) == hipSuccess && base) {
+        const uint64_t off = (uint64_t)((const char *)dev_ptr - (const char *)base);
+        if (off + (uint64_t)nbytes > (uint64_t)size)
+            return fail(KVM_ERANGE, "pool (%p) is said to hold %lld bytes but its allocation ends after %llu",
+                        dev_ptr, (long long)nbytes, (unsigned long long)((uint64_t)size - off));
+        h[kHwAllocBase] = (int64_t)(uintptr_t)base;
+        h[kHwAllocSize] = (int64_t)size;
+        if ((int64_t)size < KVM_IPC_MAX_ALLOC_BYTES) {
+            hipIpcMemHandle_t ipc;
+            if (hipIpcGetMemHandle(&ipc, base) == hipSuccess) {
+                memcpy(&h[kHwIpc], &ipc, sizeof ipc);
+                h[kHwFlags] |= kHandleHasIpc;
+            } else {
+                (void)hipGetLastError();   // stays a handle for this process only
+            }
+        }
+    } else {
+        (void)hipGetLastError();
+    }
+    h[kHwCheck] = handle_check(h);
     return KVM_OK;
 }
 
-static int open_handle(const int64_t *h, const char *what, const char **ptr, int64_t *nbytes)
+// Resolves a handle to a pointer valid in this process.  *map = local base of the other
+// process's allocation when the handle had to be opened, null for one of this process's.
+// The caller holds g_mu.
+static int open_handle(const int64_t *h, const char *what, const char **ptr, int64_t *nbytes, const char **map)
 {
     if (!h) return fail(KVM_EINVAL, "%s handle is null", what);
-    if (h[0] != kHandleMagic || h[5] != (h[0] ^ h[1] ^ h[2] ^ h[3] ^ h[4]))
+    if (h[kHwMagic] != kHandleMagic || h[kHwCheck] != handle_check(h))
         return fail(KVM_EHANDLE, "%s handle is not a kvmove memory handle", what);
-    if (h[1] != (int64_t)getpid())
-        return fail(KVM_EHANDLE,
-                    "%s handle was made by process %lld; this build resolves handles inside one process only",
-                    what, (long long)h[1]);
-    *ptr = (const char *)(uintptr_t)h[3];
-    *nbytes = h[4];
+    if (h[kHwBytes] <= 0 || h[kHwPtr] == 0)
+        return fail(KVM_EHANDLE, "%s handle names no memory", what);
+    *nbytes = h[kHwBytes];
+    *map = nullptr;
+    if (h[kHwPid] == (int64_t)getpid()) {
+        *ptr = (const char *)(uintptr_t)h[kHwPtr];
+        return KVM_OK;
+    }
+    if (!(h[kHwFlags] & kHandleHasIpc)) {
+        if (h[kHwAllocSize] >= KVM_IPC_MAX_ALLOC_BYTES)
+            return fail(KVM_EHANDLE,
+                        "%s handle of process %lld names a pool inside an allocation of %lld bytes; allocations of "
+                        "%lld bytes and more are not shared between processes",
+                        what, (long long)h[kHwPid], (long long)h[kHwAllocSize], (long long)KVM_IPC_MAX_ALLOC_BYTES);
+        return fail(KVM_EHANDLE, "%s handle of process %lld was not exported for other processes", what,
+                    (long long)h[kHwPid]);
+    }
+    const int64_t off = h[kHwPtr] - h[kHwAllocBase];
+    if (h[kHwAllocSize] <= 0 || h[kHwAllocSize] >= KVM_IPC_MAX_ALLOC_BYTES || off < 0 ||
+        off + h[kHwBytes] > h[kHwAllocSize])
+        return fail(KVM_EHANDLE, "%s handle of process %lld is inconsistent (pool at offset %lld, %lld bytes, in an "
+                    "allocation of %lld)", what, (long long)h[kHwPid], (long long)off, (long long)h[kHwBytes],
+                    (long long)h[kHwAllocSize]);
+    hipIpcMemHandle_t ipc;
+    memcpy(&ipc, &h[kHwIpc], sizeof ipc);
+    for (size_t i = 0; i < g_opened.size(); ++i) {
+        Opened &o = g_opened[i];
+        if (o.pid != h[kHwPid] || o.remote_base != h[kHwAllocBase]) continue;
+        if (o.size == h[kHwAllocSize] && memcmp(&o.handle, &ipc, sizeof ipc) == 0) {
+            *ptr = o.local_base + off;
+            *map = o.local_base;
+            return KVM_OK;
+        }
+        // The exporting process has made a new allocation at the old address: the old
+        // mapping and every pool bound through it are stale.
+        KVM_HIP(hipDeviceSynchronize());
+        for (auto it = g_sources.begin(); it != g_sources.end();)
+            it = (it->second.map_k == o.local_base || it->second.map_v == o.local_base) ? g_sources.erase(it) : ++it;
+        (void)hipIpcCloseMemHandle(o.local_base);
+        g_opened.erase(g_opened.begin() + (ptrdiff_t)i);
+        break;
+    }
+    void *local = nullptr;
+    const hipError_t e = hipIpcOpenMemHandle(&local, ipc, hipIpcMemLazyEnablePeerAccess);
+    if (e != hipSuccess || !local) {
+        (void)hipGetLastError();
+        return fail(KVM_EHANDLE, "%s handle of process %lld could not be opened: %s", what, (long long)h[kHwPid],
+                    hipGetErrorString(e));
+    }
+    g_opened.push_back(Opened{h[kHwPid], h[kHwAllocBase], h[kHwAllocSize], ipc, (char *)local});
+    *ptr = (char *)local + off;
+    *map = (char *)local;
     return KVM_OK;
 }
 
-int kvm_register_source(int32_t ctx_pp_size, int32_t ctx_tp_size, int32_t pp_rank, int32_t tp_rank,
-                        int64_t num_layers, int64_t num_kv_heads, const void *k_base,
-                        const void *v_base, int64_t nbytes_each)
+static int check_source_args(int32_t ctx_pp_size, int32_t ctx_tp_size, int32_t pp_rank, int32_t tp_rank,
+                             int64_t num_layers, int64_t num_kv_heads, const void *k_base, const void *v_base,
+                             int64_t nbytes_each)
 {
     if (!k_base || !v_base || nbytes_each <= 0)
         return fail(KVM_EINVAL, "kvm_register_source: null pool or non-positive size");
@@ -963,6 +1090,16 @@ int kvm_register_source(int32_t ctx_pp_size, int32_t ctx_tp_size, int32_t pp_ran
     if (num_layers <= 0 || num_kv_heads <= 0 || num_layers % ctx_pp_size || num_kv_heads % ctx_tp_size)
         return fail(KVM_EINVAL, "L %lld / H %lld do not split over pp %d / tp %d", (long long)num_layers,
                     (long long)num_kv_heads, ctx_pp_size, ctx_tp_size);
+    return KVM_OK;
+}
+
+int kvm_register_source(int32_t ctx_pp_size, int32_t ctx_tp_size, int32_t pp_rank, int32_t tp_rank,
+                        int64_t num_layers, int64_t num_kv_heads, const void *k_base,
+                        const void *v_base, int64_t nbytes_each, int64_t ctx_instance)
+{
+    if (int rc = check_source_args(ctx_pp_size, ctx_tp_size, pp_rank, tp_rank, num_layers, num_kv_heads, k_base,
+                                   v_base, nbytes_each))
+        return rc;
     int dk = 0, dv = 0;
     if (int rc = device_of(k_base, "context K pool", &dk)) return rc;
     if (int rc = device_of(v_base, "context V pool", &dv)) return rc;
@@ -970,23 +1107,18 @@ int kvm_register_source(int32_t ctx_pp_size, int32_t ctx_tp_size, int32_t pp_ran
     if (int rc = check_extent(k_base, (uint64_t)nbytes_each, extent_of(k_base), "context K pool")) return rc;
     if (int rc = check_extent(v_base, (uint64_t)nbytes_each, extent_of(v_base), "context V pool")) return rc;
     Source s{ctx_pp_size, ctx_tp_size, num_layers, num_kv_heads, (const char *)k_base,
-             (const char *)v_base, nbytes_each};
+             (const char *)v_base, nbytes_each, nullptr, nullptr};
     std::lock_guard<std::mutex> lock(g_mu);
-    g_sources[{pp_rank, tp_rank}] = s;
+    g_sources[SourceKey{ctx_instance, pp_rank, tp_rank}] = s;
     return KVM_OK;
 }
 
 int kvm_register_mem_handle(const int64_t *k_handle, const int64_t *v_handle, int64_t num_layers,
                             int64_t num_kv_heads, const int64_t context_pc[4],
-                            const int64_t decoding_pc[4])
+                            const int64_t decoding_pc[4], int64_t ctx_instance)
 {
     if (!context_pc || !decoding_pc) return fail(KVM_EINVAL, "parallel config list is null");
-    const char *k = nullptr, *v = nullptr;
-    int64_t kb = 0, vb = 0;
-    if (int rc = open_handle(k_handle, "K", &k, &kb)) return rc;
-    if (int rc = open_handle(v_handle, "V", &v, &vb)) return rc;
-    if (kb != vb) return fail(KVM_EMISMATCH, "K pool (%lld bytes) and V pool (%lld bytes) differ",
-                              (long long)kb, (long long)vb);
+    if (!k_handle || !v_handle) return fail(KVM_EINVAL, "a memory handle is null");
     // [tp_size, tp_rank, pp_size, pp_rank]; the decoding list only has to be well formed here,
     // the decoding rank's rectangle is taken from each migrate call.
     if (decoding_pc[0] <= 0 || decoding_pc[2] <= 0 || decoding_pc[1] < 0 || decoding_pc[1] >= decoding_pc[0] ||
@@ -994,29 +1126,81 @@ int kvm_register_mem_handle(const int64_t *k_handle, const int64_t *v_handle, in
         return fail(KVM_EINVAL, "decoding parallel config [%lld,%lld,%lld,%lld] is malformed",
                     (long long)decoding_pc[0], (long long)decoding_pc[1], (long long)decoding_pc[2],
                     (long long)decoding_pc[3]);
-    return kvm_register_source((int32_t)context_pc[2], (int32_t)context_pc[0], (int32_t)context_pc[3],
-                               (int32_t)context_pc[1], num_layers, num_kv_heads, k, v, kb);
+    for (int i = 0; i < 4; ++i)
+        if (context_pc[i] < 0 || context_pc[i] > INT32_MAX)
+            return fail(KVM_EINVAL, "context parallel config [%lld,%lld,%lld,%lld] is malformed",
+                        (long long)context_pc[0], (long long)context_pc[1], (long long)context_pc[2],
+                        (long long)context_pc[3]);
+    // Handles of this process take the same road as raw pointers.
+    if (k_handle[kHwMagic] == kHandleMagic && v_handle[kHwMagic] == kHandleMagic &&
+        k_handle[kHwPid] == (int64_t)getpid() && v_handle[kHwPid] == (int64_t)getpid()) {
+        const char *k = nullptr, *v = nullptr, *mk = nullptr, *mv = nullptr;
+        int64_t kb = 0, vb = 0;
+        if (int rc = open_handle(k_handle, "K", &k, &kb, &mk)) return rc;
+        if (int rc = open_handle(v_handle, "V", &v, &vb, &mv)) return rc;
+        if (kb != vb) return fail(KVM_EMISMATCH, "K pool (%lld bytes) and V pool (%lld bytes) differ",
+                                  (long long)kb, (long long)vb);
+        return kvm_register_source((int32_t)context_pc[2], (int32_t)context_pc[0], (int32_t)context_pc[3],
+                                   (int32_t)context_pc[1], num_layers, num_kv_heads, k, v, kb, ctx_instance);
+    }
+    std::lock_guard<std::mutex> lock(g_mu);
+    const char *k = nullptr, *v = nullptr, *mk = nullptr, *mv = nullptr;
+    int64_t kb = 0, vb = 0;
+    if (int rc = open_handle(k_handle, "K", &k, &kb, &mk)) return rc;
+    if (int rc = open_handle(v_handle, "V", &v, &vb, &mv)) return rc;
+    if (kb != vb) return fail(KVM_EMISMATCH, "K pool (%lld bytes) and V pool (%lld bytes) differ",
+                              (long long)kb, (long long)vb);
+    if (int rc = check_source_args((int32_t)context_pc[2], (int32_t)context_pc[0], (int32_t)context_pc[3],
+                                   (int32_t)context_pc[1], num_layers, num_kv_heads, k, v, kb))
+        return rc;
+    // A mapped allocation is device memory of the size its handle states: open_handle has
+    // checked that the pool lies inside it, and the runtime's own queries may not know the
+    // mapping as an allocation.
+    Source s{(int32_t)context_pc[2], (int32_t)context_pc[0], num_layers, num_kv_heads, k, v, kb, mk, mv};
+    g_sources[SourceKey{ctx_instance, (int32_t)context_pc[3], (int32_t)context_pc[1]}] = s;
+    return KVM_OK;
 }
 
 int kvm_reset(void)
 {
     std::lock_guard<std::mutex> lock(g_mu);
     g_sources.clear();
-    std::lock_guard<std::mutex> lock2(g_checked_mu);
-    g_checked.clear();
-    return KVM_OK;
+    int rc = KVM_OK;
+    if (!g_opened.empty()) {
+        // kernels in flight may still read the mappings
+        if (hipDeviceSynchronize() != hipSuccess) {
+            (void)hipGetLastError();
+            rc = fail(KVM_EHIP, "kvm_reset: the device did not become idle");
+        }
+        for (Opened &o : g_opened) {
+            const hipError_t e = hipIpcCloseMemHandle(o.local_base);
+            if (e != hipSuccess) {
+                (void)hipGetLastError();
+                rc = fail(KVM_EHIP, "hipIpcCloseMemHandle failed: %s", hipGetErrorString(e));
+            }
+        }
+        g_opened.clear();
+    }
+    return rc;
+}
+
+int64_t kvm_opened_handles(void)
+{
+    std::lock_guard<std::mutex> lock(g_mu);
+    return (int64_t)g_opened.size();
 }
 
 int kvm_migrate_plan(const KvmGeom *geom, int64_t n, const void *dst_k, const void *dst_v, int64_t out[8])
 {
     if (!out) return fail(KVM_EINVAL, "out is null");
+    if (n < 0) return fail(KVM_EINVAL, "n is negative");
     Plan plan;
-    if (int rc = build_plan(geom, dst_k, dst_v, &plan)) return rc;
-    int64_t launches = 0, wgs = 0;
+    if (int rc = build_plan(geom, dst_k, dst_v, &plan, !dst_k && !dst_v)) return rc;
+    int64_t launches = 0, wgs = 0, max_items = 0;
     int threads = 0;
     bool simple = false;
     if (int rc = launch_copy(plan.segs, nullptr, n, nullptr, nullptr, plan.dst_block_stride, plan.vec,
-                             nullptr, &launches, &wgs, &threads, 0, &simple))
+                             nullptr, &launches, &wgs, &threads, 0, &simple, &max_items))
         return rc;
     out[0] = wgs;
     out[1] = threads;
@@ -1025,7 +1209,7 @@ int kvm_migrate_plan(const KvmGeom *geom, int64_t n, const void *dst_k, const vo
     out[4] = launches;
     out[5] = plan.payload_per_block;
     out[6] = simple ? 1 : 0;
-    out[7] = 0;
+    out[7] = max_items;
     return KVM_OK;
 }
 

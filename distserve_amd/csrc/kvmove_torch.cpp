@@ -49,25 +49,38 @@ std::vector<int64_t> get_ipc_mem_handle(const at::Tensor &t)
     return h;
 }
 
-void register_ipc_mem_handle(std::vector<int64_t> k_handle, std::vector<int64_t> v_handle,
-                             int64_t num_layers, int64_t num_heads,
-                             std::vector<int64_t> context_parallel_config,
-                             std::vector<int64_t> decoding_parallel_config)
+// The *_from forms (no counterpart in the reference) name the context instance whose pools
+// are bound or read, for a process that serves more than one; the reference's own schemas
+// below them mean instance 0.
+void register_ipc_mem_handle_from(int64_t context_instance, std::vector<int64_t> k_handle,
+                                  std::vector<int64_t> v_handle, int64_t num_layers, int64_t num_heads,
+                                  std::vector<int64_t> context_parallel_config,
+                                  std::vector<int64_t> decoding_parallel_config)
 {
     TORCH_CHECK(k_handle.size() == KVM_HANDLE_WORDS && v_handle.size() == KVM_HANDLE_WORDS,
                 "register_ipc_mem_handle: a memory handle has ", KVM_HANDLE_WORDS, " words");
     TORCH_CHECK(context_parallel_config.size() == 4 && decoding_parallel_config.size() == 4,
                 "register_ipc_mem_handle: parallel configs are [tp_size, tp_rank, pp_size, pp_rank]");
     check(kvm_register_mem_handle(k_handle.data(), v_handle.data(), num_layers, num_heads,
-                                  context_parallel_config.data(), decoding_parallel_config.data()),
+                                  context_parallel_config.data(), decoding_parallel_config.data(),
+                                  context_instance),
           "register_ipc_mem_handle");
 }
 
-void migrate_blocks(int64_t context_pp_size, int64_t context_tp_size,
-                    std::vector<int64_t> context_block_indexes, int64_t decoding_pp_size,
-                    int64_t decoding_tp_size, int64_t decoding_pp_rank, int64_t decoding_tp_rank,
-                    std::vector<int64_t> decoding_block_indexes, const at::Tensor &k_cache,
-                    const at::Tensor &v_cache)
+void register_ipc_mem_handle(std::vector<int64_t> k_handle, std::vector<int64_t> v_handle,
+                             int64_t num_layers, int64_t num_heads,
+                             std::vector<int64_t> context_parallel_config,
+                             std::vector<int64_t> decoding_parallel_config)
+{
+    register_ipc_mem_handle_from(0, std::move(k_handle), std::move(v_handle), num_layers, num_heads,
+                                 std::move(context_parallel_config), std::move(decoding_parallel_config));
+}
+
+void migrate_blocks_from(int64_t context_instance, int64_t context_pp_size, int64_t context_tp_size,
+                         std::vector<int64_t> context_block_indexes, int64_t decoding_pp_size,
+                         int64_t decoding_tp_size, int64_t decoding_pp_rank, int64_t decoding_tp_rank,
+                         std::vector<int64_t> decoding_block_indexes, const at::Tensor &k_cache,
+                         const at::Tensor &v_cache)
 {
     check_pool(k_cache, "k_cache", true);
     check_pool(v_cache, "v_cache", true);
@@ -92,10 +105,22 @@ void migrate_blocks(int64_t context_pp_size, int64_t context_tp_size,
     g.dec_tp_size = (int32_t)decoding_tp_size;
     g.dec_pp_rank = (int32_t)decoding_pp_rank;
     g.dec_tp_rank = (int32_t)decoding_tp_rank;
+    g.ctx_instance = context_instance;
     check(kvm_migrate(&g, context_block_indexes.data(), decoding_block_indexes.data(),
                       (int64_t)context_block_indexes.size(), k_cache.data_ptr(), v_cache.data_ptr(),
                       k_cache.size(0), current_stream(k_cache)),
           "migrate_blocks");
+}
+
+void migrate_blocks(int64_t context_pp_size, int64_t context_tp_size,
+                    std::vector<int64_t> context_block_indexes, int64_t decoding_pp_size,
+                    int64_t decoding_tp_size, int64_t decoding_pp_rank, int64_t decoding_tp_rank,
+                    std::vector<int64_t> decoding_block_indexes, const at::Tensor &k_cache,
+                    const at::Tensor &v_cache)
+{
+    migrate_blocks_from(0, context_pp_size, context_tp_size, std::move(context_block_indexes), decoding_pp_size,
+                        decoding_tp_size, decoding_pp_rank, decoding_tp_rank, std::move(decoding_block_indexes),
+                        k_cache, v_cache);
 }
 
 void swap(std::vector<int64_t> source_block_ids, std::vector<int64_t> target_block_ids, bool is_swap_in,
@@ -145,6 +170,13 @@ KVM_TORCH_LIBRARY(KVM_MIGRATION_NS, m)
           "int decoding_pp_size, int decoding_tp_size, int decoding_pp_rank, int decoding_tp_rank, "
           "int[] decoding_block_indexes, Tensor k_cache, Tensor v_cache) -> ()",
           migrate_blocks);
+    m.def("register_ipc_mem_handle_from(int context_instance, int[] k_handle, int[] v_handle, int num_layers, "
+          "int num_heads, int[] context_parallel_config, int[] decoding_parallel_config) -> ()",
+          register_ipc_mem_handle_from);
+    m.def("migrate_blocks_from(int context_instance, int context_pp_size, int context_tp_size, "
+          "int[] context_block_indexes, int decoding_pp_size, int decoding_tp_size, int decoding_pp_rank, "
+          "int decoding_tp_rank, int[] decoding_block_indexes, Tensor k_cache, Tensor v_cache) -> ()",
+          migrate_blocks_from);
 }
 
 KVM_TORCH_LIBRARY(KVM_SWAP_NS, m)

@@ -66,8 +66,9 @@ class SingleStageLLMEngine:
 class ContextStageLLMEngine(SingleStageLLMEngine):
     stage = Stage.CONTEXT
 
-    def __init__(self, *args, **kwargs):
+    def __init__(self, *args, instance_id: int = 0, **kwargs):
         super().__init__(*args, **kwargs)
+        self.instance_id = instance_id   # names this instance's pools on the decoding side
         self.bridge_queue: List[MigratingRequest] = []
         self.scheduler = None     # optional ContextStageFCFSScheduler, told when a request has left
 
@@ -75,7 +76,7 @@ class ContextStageLLMEngine(SingleStageLLMEngine):
         """Tail of the context step: the request's blocks stay where they are and their
         table travels to the decoding instance (reference :393-401)."""
         migrating_req = MigratingRequest(request, self.block_manager.get_block_table(request.request_id),
-                                         self.parallel_config)
+                                         self.parallel_config, self.instance_id)
         self.bridge_queue.append(migrating_req)
         return migrating_req
 
@@ -101,6 +102,7 @@ class DecodingStageLLMEngine(SingleStageLLMEngine):
         # True: MigrationEnd is stamped after the copy's event has completed on the GPU
         self.gpu_complete_lifetime_events = gpu_complete_lifetime_events
         self.lifetime_events: Dict[int, List[LifetimeEvent]] = {}
+        self._release_takes_events: Optional[bool] = None
 
     def _lifetime(self, request_id: int, event_type: LifetimeEventType) -> None:
         event = LifetimeEvent(event_type)
@@ -121,11 +123,21 @@ class DecodingStageLLMEngine(SingleStageLLMEngine):
         return self.lifetime_events.pop(request_id, [])
 
     def register_kvcache_mem_handles(self, context_parallel_config: ParallelConfig,
-                                     kv_cache_mem_handles: List[List[Tuple[MemoryHandle, MemoryHandle]]]) -> None:
-        """Hand the context instance's handles to every decoding worker (reference :469-483)."""
+                                     kv_cache_mem_handles: List[List[Tuple[MemoryHandle, MemoryHandle]]],
+                                     context_instance: int = 0) -> None:
+        """Hand a context instance's handles to every decoding worker (reference :469-483)."""
         self.kv_cache_mem_handles = kv_cache_mem_handles
-        self._remote_call_all_workers_async("register_kvcache_mem_handles", context_parallel_config,
-                                            kv_cache_mem_handles)
+        if context_instance:
+            self._remote_call_all_workers_async("register_kvcache_mem_handles", context_parallel_config,
+                                                kv_cache_mem_handles, context_instance)
+        else:
+            self._remote_call_all_workers_async("register_kvcache_mem_handles", context_parallel_config,
+                                                kv_cache_mem_handles)
+
+    def _call_migrate(self, ctx_idx: List[int], config: ParallelConfig, dec_idx: List[int], instance: int) -> None:
+        # the reference's three-argument call unless a second context instance is in play
+        extra = (instance,) if instance else ()
+        self._remote_call_all_workers_async("migrate_blocks", ctx_idx, config, dec_idx, *extra)
 
     def _allocate_for_migration(self, migrating_req: MigratingRequest) -> List[int]:
         """Blocks on this side for the request's *prompt* (reference :505-517)."""
@@ -144,13 +156,36 @@ class DecodingStageLLMEngine(SingleStageLLMEngine):
             f"{len(target_block_indexes)} decoding blocks")
         return target_block_indexes
 
+    def _callback_takes_events(self) -> bool:
+        """Whether the release callback has a ``migrate_events`` parameter; the reference's
+        (``clear_migrated_blocks_callback(migrated_request)``, :405-410) has not."""
+        if self._release_takes_events is None:
+            import inspect
+
+            try:
+                params = inspect.signature(self.clear_migrated_blocks_callback).parameters
+                self._release_takes_events = "migrate_events" in params or any(
+                    p.kind is inspect.Parameter.VAR_KEYWORD for p in params.values())
+            except (TypeError, ValueError):
+                self._release_takes_events = False
+        return self._release_takes_events
+
     def _release_source_blocks(self, migrating_reqs: List[MigratingRequest]) -> None:
         if self.clear_migrated_blocks_callback is None:
             return
         events = [w.latest_migrate_event for row in self.workers for w in row
                   if getattr(w, "latest_migrate_event", None) is not None]
+        if self._callback_takes_events():
+            for migrating_req in migrating_reqs:
+                self.clear_migrated_blocks_callback(migrating_req, migrate_events=events)
+            return
+        # A callback of the reference's shape cannot order the context instance's later work
+        # behind the copies, so the blocks are released only once the copies have finished.
+        for event in events:
+            if hasattr(event, "synchronize"):
+                event.synchronize()
         for migrating_req in migrating_reqs:
-            self.clear_migrated_blocks_callback(migrating_req, events)
+            self.clear_migrated_blocks_callback(migrating_req)
 
     def _migrate_blocks(self, migrating_req: MigratingRequest) -> None:
         """Move one request from the context instance to this one (reference :490-536):
@@ -159,8 +194,8 @@ class DecodingStageLLMEngine(SingleStageLLMEngine):
         req = migrating_req.req
         target_block_indexes = self._allocate_for_migration(migrating_req)
         self._lifetime(req.request_id, LifetimeEventType.MigrationBegin)
-        self._remote_call_all_workers_async("migrate_blocks", migrating_req.block_indexes,
-                                            migrating_req.context_parallel_config, target_block_indexes)
+        self._call_migrate(migrating_req.block_indexes, migrating_req.context_parallel_config,
+                           target_block_indexes, getattr(migrating_req, "context_instance", 0))
         self._wait_for_copies()
         self._lifetime(req.request_id, LifetimeEventType.MigrationEnd)
         self._release_source_blocks([migrating_req])
@@ -177,7 +212,9 @@ class DecodingStageLLMEngine(SingleStageLLMEngine):
         if not migrating_reqs:
             return
         config = migrating_reqs[0].context_parallel_config
-        assert all(m.context_parallel_config.to_list()[0::2] == config.to_list()[0::2] for m in migrating_reqs), \
+        instance = getattr(migrating_reqs[0], "context_instance", 0)
+        assert all(m.context_parallel_config.to_list()[0::2] == config.to_list()[0::2]
+                   and getattr(m, "context_instance", 0) == instance for m in migrating_reqs), \
             "requests migrated together must come from one context instance"
         ctx_idx: List[int] = []
         dec_idx: List[int] = []
@@ -190,7 +227,7 @@ class DecodingStageLLMEngine(SingleStageLLMEngine):
             ctx_idx += m.block_indexes
             dec_idx += target
             self._lifetime(rid, LifetimeEventType.MigrationBegin)
-        self._remote_call_all_workers_async("migrate_blocks", ctx_idx, config, dec_idx)
+        self._call_migrate(ctx_idx, config, dec_idx, instance)
         self._wait_for_copies()
         for m in migrating_reqs:
             self._lifetime(m.req.request_id, LifetimeEventType.MigrationEnd)

@@ -87,7 +87,10 @@ class MigratingRequest:
     """Element of the bridge queue between the two instances (reference request.py:408-433):
     a request that finished prefill, whose blocks still sit in the context instance's pools."""
 
-    def __init__(self, req: Request, block_indexes: List[int], context_parallel_config: ParallelConfig):
+    def __init__(self, req: Request, block_indexes: List[int], context_parallel_config: ParallelConfig,
+                 context_instance: int = 0):
         self.req = req
         self.block_indexes = block_indexes
         self.context_parallel_config = context_parallel_config
+        # which context instance holds the blocks (not in the reference, which has one)
+        self.context_instance = context_instance

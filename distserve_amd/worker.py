@@ -133,25 +133,29 @@ class Worker:
     # ---- migration
 
     def register_kvcache_mem_handles(self, context_parallel_config: ParallelConfig,
-                                     kvcache_ipc_mem_handles: List[List[Tuple[MemoryHandle, MemoryHandle]]]) -> None:
+                                     kvcache_ipc_mem_handles: List[List[Tuple[MemoryHandle, MemoryHandle]]],
+                                     context_instance: int = 0) -> None:
         """Bind every context rank's pools, ``handles[pp_rank][tp_rank] = (k, v)``
-        (reference worker.py:229-248)."""
+        (reference worker.py:229-248).  The handles may come from another process: they are
+        plain lists of ints.  ``context_instance`` (not in the reference, where a decoding
+        worker serves one context instance) keeps several instances' pools apart."""
         for pp_rank, stage_handles in enumerate(kvcache_ipc_mem_handles):
             for tp_rank, (k_handle, v_handle) in enumerate(stage_handles):
                 rank_config = copy.deepcopy(context_parallel_config)
                 rank_config.pipeline_parallel_rank = pp_rank
                 rank_config.tensor_parallel_rank = tp_rank
-                torch.ops.block_migration_ops.register_ipc_mem_handle(
-                    k_handle, v_handle,
+                torch.ops.block_migration_ops.register_ipc_mem_handle_from(
+                    context_instance, k_handle, v_handle,
                     self.model_config.get_num_layers(), self.model_config.get_num_heads(),
                     rank_config.to_list(), self.parallel_config.to_list())
         torch.cuda.synchronize()
 
     def migrate_blocks(self, context_block_indexes: List[int], context_parallel_config: ParallelConfig,
-                       decoding_block_indexes: List[int]) -> None:
+                       decoding_block_indexes: List[int], context_instance: int = 0) -> None:
         """Pull this rank's share of the listed context blocks into its own pools, on the
         current stream, without waiting for the GPU (reference worker.py:250-267)."""
-        torch.ops.block_migration_ops.migrate_blocks(
+        torch.ops.block_migration_ops.migrate_blocks_from(
+            context_instance,
             context_parallel_config.pipeline_parallel_size,
             context_parallel_config.tensor_parallel_size,
             context_block_indexes,

@@ -39,10 +39,14 @@ extern "C" {
 #define KVM_EDUP (-3)       /* a destination block index occurs twice in one call */
 #define KVM_ENOTREG (-4)    /* a context rank the copy needs was never registered */
 #define KVM_EHIP (-5)       /* a HIP runtime call failed */
-#define KVM_EHANDLE (-6)    /* memory handle is not one of this process's */
+#define KVM_EHANDLE (-6)    /* memory handle is malformed, or cannot be opened in this process */
 #define KVM_EMISMATCH (-7)  /* registered pools disagree with the call's geometry */
 
-#define KVM_HANDLE_WORDS 8  /* int64 words in a memory handle */
+#define KVM_HANDLE_WORDS 17 /* int64 words in a memory handle */
+
+/* Device allocations of this size and above are not exported to other processes: the
+ * handle of such a pool still works inside the process that made it. */
+#define KVM_IPC_MAX_ALLOC_BYTES (2147483648LL)
 
 /* Whole-model KV geometry and both instances' layouts for one migrate call.
  * The [tp_size, tp_rank, pp_size, pp_rank] order of ParallelConfig.to_list()
@@ -59,6 +63,8 @@ typedef struct KvmGeom {
     int32_t dec_tp_size;
     int32_t dec_pp_rank;   /* ... and the decoding rank that pulls */
     int32_t dec_tp_rank;
+    int64_t ctx_instance;  /* which context instance's registered pools are read (0 = the only
+                              one, as in the reference, where a decoding worker has one) */
 } KvmGeom;
 
 /* Library version: major*10000 + minor*100 + patch. */
@@ -69,10 +75,17 @@ const char *kvm_last_error(void);
 
 /*
  * Replaces torch.ops.block_migration_ops.get_ipc_mem_handle(tensor)
- * (distserve/worker.py:133-134).  Writes an opaque KVM_HANDLE_WORDS-word token naming
- * the device allocation [dev_ptr, dev_ptr + nbytes).  Single-GPU build: the token is
- * valid only inside the process that made it (same-process pointer registry); a token
- * from another process is refused with KVM_EHANDLE.
+ * (distserve/worker.py:133-134).  Writes an opaque KVM_HANDLE_WORDS-word handle naming
+ * the device memory [dev_ptr, dev_ptr + nbytes): the exporting process, the pointer, and a
+ * hipIpcMemHandle_t of the device allocation that holds it together with the pool's offset
+ * inside that allocation (a pool may be a piece of a larger allocation, as with torch's
+ * caching allocator).  The words are plain data: send them to the decoding worker by any
+ * means.  Inside the exporting process the handle resolves to the pointer itself (a
+ * process cannot open its own IPC handle); in another process registration maps the
+ * allocation with hipIpcOpenMemHandle.  An allocation of KVM_IPC_MAX_ALLOC_BYTES or more,
+ * or one the runtime cannot export, yields a handle that is valid in its own process
+ * only; another process that registers it gets KVM_EHANDLE and the reason.  The exporting
+ * process must keep the allocation alive while any process uses the handle.
  */
 int kvm_get_mem_handle(const void *dev_ptr, int64_t nbytes, int64_t *out_handle);
 
@@ -82,19 +95,32 @@ int kvm_get_mem_handle(const void *dev_ptr, int64_t nbytes, int64_t *out_handle)
  * (distserve/worker.py:239-246).  Binds context rank (pp_rank, tp_rank)'s K and V pools.
  * context_pc / decoding_pc are [tp_size, tp_rank, pp_size, pp_rank]
  * (distserve/config.py:57-63).  Registering the same rank again replaces the binding.
+ * Handles made by another process are opened here (hipIpcOpenMemHandle, once per
+ * allocation and process, however many pools lie in it) and stay mapped until kvm_reset.
+ * ctx_instance (no counterpart in the reference, whose decoding worker serves a single
+ * context instance) keeps the pools of several context instances apart in one process:
+ * bindings are keyed by (ctx_instance, pp_rank, tp_rank), and a migrate call reads the
+ * instance its geometry names.  Pass 0 where there is one.
  */
 int kvm_register_mem_handle(const int64_t *k_handle, const int64_t *v_handle,
                             int64_t num_layers, int64_t num_kv_heads,
-                            const int64_t context_pc[4], const int64_t decoding_pc[4]);
+                            const int64_t context_pc[4], const int64_t decoding_pc[4],
+                            int64_t ctx_instance);
 
-/* Same binding from raw device pointers (no handle round trip). */
+/* Same binding from raw device pointers of this process (no handle round trip). */
 int kvm_register_source(int32_t ctx_pp_size, int32_t ctx_tp_size, int32_t pp_rank, int32_t tp_rank,
                         int64_t num_layers, int64_t num_kv_heads,
-                        const void *k_base, const void *v_base, int64_t nbytes_each);
+                        const void *k_base, const void *v_base, int64_t nbytes_each,
+                        int64_t ctx_instance);
 
-/* Forget every registered context pool (the reference has no counterpart: its
- * registry lives as long as the worker process; tests and benches need a clean slate). */
+/* Forget every registered context pool of every instance and unmap every allocation
+ * opened from another process, after the device has finished the work in flight (the
+ * reference has no counterpart: its registry lives as long as the worker process; tests,
+ * benches and a worker that re-binds to a restarted context instance need a clean slate). */
 int kvm_reset(void);
+
+/* Allocations of other processes currently mapped by registration (for tests and reports). */
+int64_t kvm_opened_handles(void);
 
 /*
  * Replaces torch.ops.block_migration_ops.migrate_blocks(...)
@@ -170,8 +196,12 @@ int64_t kvm_get_option(const char *name);
  * reports: out[0] = workgroups per block (K and V together), out[1] = workgroup size,
  * out[2] = vector width in bytes, out[3] = number of source segments,
  * out[4] = kernel launches, out[5] = payload bytes per block (K+V, this rank's share),
- * out[6] = 1 when the short-prologue kernel (kvm_copy_simple_kernel) serves the shape, out[7] = 0.
- * Needs the sources registered (alignment of their bases picks the vector width).
+ * out[6] = 1 when the short-prologue kernel (kvm_copy_simple_kernel) serves the shape,
+ * out[7] = work-items (workgroups x workgroup size) of the largest launch, which the
+ * library keeps below 2^32 by splitting the block list over more launches.
+ * Needs the sources registered (alignment of their bases picks the vector width), except
+ * with dst_k == dst_v == NULL: then the plan is pure arithmetic, touches no device, and
+ * takes every pool for 16-byte aligned.
  */
 int kvm_migrate_plan(const KvmGeom *geom, int64_t n, const void *dst_k, const void *dst_v,
                      int64_t out[8]);

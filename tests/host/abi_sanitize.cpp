@@ -77,6 +77,45 @@ int main()
     int64_t plan[8];
     EXPECT(kvm_migrate_plan(&g, 10, fake_k, fake_v, nullptr) == KVM_EINVAL);
     EXPECT(kvm_migrate_plan(&g, 10, fake_k, fake_v, plan) == KVM_ENOTREG);
+    KvmGeom other = g;
+    other.ctx_instance = 3;                                     // no instance has anything registered
+    EXPECT(kvm_migrate_plan(&other, 10, fake_k, fake_v, plan) == KVM_ENOTREG);
+
+    // Launch sizes, as pure arithmetic (null pools: nothing registered, no device touched).
+    // A launch is 2 * tiles * blocks workgroups of 64 lanes and must stay below 2^32 work-items,
+    // so big blocks get fewer index pairs per launch instead of a launch the runtime refuses.
+    EXPECT(kvm_migrate_plan(&g, -1, nullptr, nullptr, plan) == KVM_EINVAL);
+    {
+        // LLaMA-2-7B 1 -> 1: 4 MiB per pool kind per block = 4096 tiles, 432 blocks per launch
+        KvmGeom g7 = geom(32, 32, 16, 128, 2);
+        EXPECT(kvm_migrate_plan(&g7, 909, nullptr, nullptr, plan) == KVM_OK);
+        EXPECT(plan[0] == 8192 && plan[1] == 64 && plan[2] == 16 && plan[3] == 1 && plan[4] == 3 && plan[6] == 1);
+        EXPECT(plan[5] == 8388608);
+        EXPECT(plan[7] == 2ll * 4096 * 432 * 64);
+        // a 1 GiB block per pool kind (L 128 x H 128 x B 256 x D 128 x 2 bytes): 2^20 tiles, so at
+        // most 31 blocks fit a launch (2 * 31 * 2^20 * 64 < 2^32 <= 2 * 32 * 2^20 * 64)
+        KvmGeom big = geom(128, 128, 256, 128, 2);
+        for (int64_t n : {1, 31, 32, 100, 432, 1000}) {
+            EXPECT(kvm_migrate_plan(&big, n, nullptr, nullptr, plan) == KVM_OK);
+            EXPECT(plan[5] == 2ll << 30);
+            EXPECT(plan[7] > 0 && plan[7] < (1ll << 32));
+            EXPECT(plan[4] == (n + 30) / 31);
+            EXPECT(plan[7] == 2ll * (1 << 20) * (n < 31 ? n : 31) * 64);
+        }
+        // the same through two context ranks whose head split does not nest (general kernel, 2 segments)
+        KvmGeom big2 = geom(128, 128, 256, 128, 2, 1, 2);
+        EXPECT(kvm_migrate_plan(&big2, 100, nullptr, nullptr, plan) == KVM_OK);
+        EXPECT(plan[3] == 2 && plan[6] == 0 && plan[7] < (1ll << 32) && plan[4] == 4);
+        // larger workgroups leave room for fewer tiles per launch
+        EXPECT(kvm_set_option("threads", 1024) == KVM_OK && kvm_set_option("unroll", 4) == KVM_OK);
+        EXPECT(kvm_migrate_plan(&big, 1000, nullptr, nullptr, plan) == KVM_OK);
+        EXPECT(plan[1] == 1024 && plan[7] < (1ll << 32));
+        EXPECT(kvm_set_option("threads", 64) == KVM_OK && kvm_set_option("unroll", 1) == KVM_OK);
+        // many small blocks: every launch of 432 pairs is far below the limit
+        KvmGeom small = geom(2, 2, 16, 8, 2);
+        EXPECT(kvm_migrate_plan(&small, 100000, nullptr, nullptr, plan) == KVM_OK);
+        EXPECT(plan[4] == (100000 + 431) / 432 && plan[7] < (1ll << 32));
+    }
 
     // handles and registration
     int64_t h[KVM_HANDLE_WORDS] = {0};
@@ -85,18 +124,48 @@ int main()
     EXPECT(kvm_get_mem_handle(fake_k, 0, h) == KVM_EINVAL);
     EXPECT(kvm_get_mem_handle(fake_k, 16, nullptr) == KVM_EINVAL);
     EXPECT(kvm_get_mem_handle(fake_k, 16, h) == KVM_EINVAL);    // host memory (or no device at all) is no pool
-    EXPECT(kvm_register_mem_handle(h, h, 4, 4, pc, pc) == KVM_EHANDLE);
-    EXPECT(kvm_register_mem_handle(nullptr, h, 4, 4, pc, pc) == KVM_EINVAL);
-    EXPECT(kvm_register_mem_handle(h, h, 4, 4, nullptr, pc) == KVM_EINVAL);
-    h[0] = 0x4b564d4f56453031LL; h[1] = 1; h[2] = 0; h[3] = 4096; h[4] = 64;   // plausible but forged: checksum missing
-    EXPECT(kvm_register_mem_handle(h, h, 4, 4, pc, pc) == KVM_EHANDLE);
-    h[5] = h[0] ^ h[1] ^ h[2] ^ h[3] ^ h[4];                                   // well formed, other process (pid 1)
-    EXPECT(kvm_register_mem_handle(h, h, 4, 4, pc, pc) == KVM_EHANDLE);
-    (void)bad_pc;
-    EXPECT(kvm_register_source(1, 1, 0, 0, 4, 4, nullptr, fake_v, 64) == KVM_EINVAL);
-    EXPECT(kvm_register_source(1, 1, 1, 0, 4, 4, fake_k, fake_v, 64) == KVM_EINVAL);
-    EXPECT(kvm_register_source(2, 1, 0, 0, 5, 4, fake_k, fake_v, 64) == KVM_EINVAL);
-    EXPECT(kvm_register_source(1, 1, 0, 0, 4, 4, fake_k, fake_v, 64) == KVM_EINVAL);   // not device memory
+    EXPECT(kvm_register_mem_handle(h, h, 4, 4, pc, pc, 0) == KVM_EHANDLE);
+    EXPECT(kvm_register_mem_handle(nullptr, h, 4, 4, pc, pc, 0) == KVM_EINVAL);
+    EXPECT(kvm_register_mem_handle(h, h, 4, 4, nullptr, pc, 0) == KVM_EINVAL);
+    EXPECT(kvm_register_mem_handle(h, h, 4, 4, pc, bad_pc, 0) == KVM_EINVAL);
+    h[0] = 0x4b564d4f56453032LL; h[1] = 1; h[2] = 0; h[3] = 4096; h[4] = 64;   // plausible but forged: checksum missing
+    EXPECT(kvm_register_mem_handle(h, h, 4, 4, pc, pc, 0) == KVM_EHANDLE);
+    EXPECT(std::strstr(kvm_last_error(), "not a kvmove memory handle") != nullptr);
+    // well-formed handles of another process (pid 1), with the checksum word as the library computes it
+    auto seal = [](int64_t *w) {
+        uint64_t x = 0x5a5a5a5a5a5a5a5aull;
+        for (int i = 0; i < KVM_HANDLE_WORDS - 1; ++i) x = ((x << 7) | (x >> 57)) ^ (uint64_t)w[i];
+        w[KVM_HANDLE_WORDS - 1] = (int64_t)x;
+    };
+    h[5] = 4096; h[6] = 1 << 20; h[7] = 0;                      // made without an IPC part
+    seal(h);
+    EXPECT(kvm_register_mem_handle(h, h, 4, 4, pc, pc, 0) == KVM_EHANDLE);
+    EXPECT(std::strstr(kvm_last_error(), "was not exported for other processes") != nullptr);
+    h[6] = 3ll << 30;                                           // inside a 3 GiB allocation: never shared
+    seal(h);
+    EXPECT(kvm_register_mem_handle(h, h, 4, 4, pc, pc, 0) == KVM_EHANDLE);
+    EXPECT(std::strstr(kvm_last_error(), "are not shared between processes") != nullptr);
+    h[7] = 1;                                                   // claims an IPC part all the same
+    seal(h);
+    EXPECT(kvm_register_mem_handle(h, h, 4, 4, pc, pc, 0) == KVM_EHANDLE);
+    EXPECT(std::strstr(kvm_last_error(), "inconsistent") != nullptr);
+    h[6] = 32;                                                  // pool of 64 bytes in an allocation of 32
+    seal(h);
+    EXPECT(kvm_register_mem_handle(h, h, 4, 4, pc, pc, 0) == KVM_EHANDLE);
+    EXPECT(std::strstr(kvm_last_error(), "inconsistent") != nullptr);
+    h[5] = 8192;                                                // pool below its allocation
+    h[6] = 1 << 20;
+    seal(h);
+    EXPECT(kvm_register_mem_handle(h, h, 4, 4, pc, pc, 0) == KVM_EHANDLE);
+    EXPECT(std::strstr(kvm_last_error(), "inconsistent") != nullptr);
+    h[4] = 0;                                                   // names no memory
+    seal(h);
+    EXPECT(kvm_register_mem_handle(h, h, 4, 4, pc, pc, 0) == KVM_EHANDLE);
+    EXPECT(kvm_opened_handles() == 0);
+    EXPECT(kvm_register_source(1, 1, 0, 0, 4, 4, nullptr, fake_v, 64, 0) == KVM_EINVAL);
+    EXPECT(kvm_register_source(1, 1, 1, 0, 4, 4, fake_k, fake_v, 64, 0) == KVM_EINVAL);
+    EXPECT(kvm_register_source(2, 1, 0, 0, 5, 4, fake_k, fake_v, 64, 0) == KVM_EINVAL);
+    EXPECT(kvm_register_source(1, 1, 0, 0, 4, 4, fake_k, fake_v, 64, 7) == KVM_EINVAL);   // not device memory
     EXPECT(kvm_reset() == KVM_OK);
 
     // swap and plain copy argument checks

@@ -90,11 +90,40 @@ def test_argument_errors_need_no_gpu(kvm, fresh_registry):
     assert e.value.code == kvm.KVM_ENOTREG
     kvm.migrate(g, [], [], 4096, 8192, 4)                       # an empty list is a no-op even then
     with pytest.raises(kvm.KvmError) as e:
-        kvm.register_mem_handle([0] * 8, [0] * 8, 4, 4, [1, 0, 1, 0], [1, 0, 1, 0])
+        kvm.register_mem_handle([0] * kvm.KVM_HANDLE_WORDS, [0] * kvm.KVM_HANDLE_WORDS, 4, 4, [1, 0, 1, 0], [1, 0, 1, 0])
     assert e.value.code == kvm.KVM_EHANDLE
     with pytest.raises(kvm.KvmError) as e:
         kvm.swap([0], [0], True, 0, 0, 0, 0, 64, 1, 1)
     assert e.value.code == kvm.KVM_EINVAL
+
+
+def test_launches_stay_below_the_grid_limit_for_blocks_of_any_size(kvm, fresh_registry):
+    """A launch is 2 x tiles x blocks workgroups of `threads` lanes; the runtime refuses 2^32
+    work-items and more, so the block list is split over more launches before anything is
+    enqueued.  Pure arithmetic: null pools, nothing registered, no device."""
+    plan = kvm.migrate_plan(kvm.geom(32, 32, 16, 128, 2), 909, 0, 0)          # LLaMA-2-7B, 1 -> 1
+    assert plan["launches"] == 3 and plan["simple_kernel"] == 1 and plan["max_work_items"] == 2 * 4096 * 432 * 64
+    big = kvm.geom(128, 128, 256, 128, 2)                                      # 1 GiB per pool kind per block
+    tiles = (1 << 30) // 1024
+    for n in (1, 31, 32, 433, 5000):
+        plan = kvm.migrate_plan(big, n, 0, 0)
+        per_launch = (2**32 - 1) // (2 * 64) // tiles                          # 31, short of the padding allowance
+        assert plan["payload_bytes_per_block"] == 2 << 30
+        assert plan["launches"] == -(-n // per_launch)
+        assert 0 < plan["max_work_items"] < 2**32
+    for threads, unroll in ((256, 4), (1024, 4)):
+        kvm.set_option("threads", threads)
+        kvm.set_option("unroll", unroll)
+        try:
+            plan = kvm.migrate_plan(big, 5000, 0, 0)
+            assert plan["threads"] == threads and 0 < plan["max_work_items"] < 2**32
+        finally:
+            kvm.set_option("threads", 64)
+            kvm.set_option("unroll", 1)
+    # with real (non-null) destination pointers the plan wants the sources registered, as before
+    with pytest.raises(kvm.KvmError) as e:
+        kvm.migrate_plan(big, 4, 4096, 8192)
+    assert e.value.code == kvm.KVM_ENOTREG
 
 
 def test_torch_ops_are_registered_with_the_reference_argument_order():
@@ -113,6 +142,11 @@ def test_torch_ops_are_registered_with_the_reference_argument_order():
     order = ["k_handle", "v_handle", "num_layers", "num_heads", "context_parallel_config", "decoding_parallel_config"]
     assert [s.index(a) for a in order] == sorted(s.index(a) for a in order)
     assert "int[]" in str(torch.ops.block_migration_ops.get_ipc_mem_handle.default._schema)
+    # the forms that name a context instance are the same schemas behind one leading argument
+    for name in ("register_ipc_mem_handle", "migrate_blocks"):
+        plain = str(getattr(torch.ops.block_migration_ops, name).default._schema).split("(", 1)[1]
+        named = str(getattr(torch.ops.block_migration_ops, name + "_from").default._schema).split("(", 1)[1]
+        assert named == "int context_instance, " + plain
     # no CPU fallback: a CPU tensor is refused, loudly
     z = torch.zeros(2, 1, 1, 2, 2, dtype=torch.float16)
     with pytest.raises(RuntimeError, match="GPU"):

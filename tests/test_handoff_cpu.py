@@ -129,3 +129,65 @@ def test_lifetime_events_keep_the_reference_json_shape(engines):
                                                    "migration_end", "decoding_begin", "decoding_end"]
     assert transmission_seconds([LifetimeEvent(LifetimeEventType.MigrationBegin, 1.0),
                                  LifetimeEvent(LifetimeEventType.MigrationEnd, 1.5)]) == 0.5
+
+
+def test_a_release_callback_of_the_reference_shape_is_called_after_the_copies(engines):
+    """The reference's callback takes the migrated request only (single_stage_engine.py:405-410).
+    It cannot be told which copies to order its later work behind, so the decoding engine
+    waits for them itself before it calls."""
+    ctx, dec = engines
+    waited, seen = [], []
+
+    class FakeEvent:
+        def __init__(self, tag):
+            self.tag = tag
+
+        def synchronize(self):
+            waited.append(self.tag)
+
+    def reference_shaped(migrated_request):
+        seen.append((migrated_request.req.request_id, list(waited)))
+
+    dec2 = DecodingStageLLMEngine(dec.model_config, dec.parallel_config, dec.cache_config, worker_factory=FakeWorker,
+                                  clear_migrated_blocks_callback=reference_shaped)
+    dec2._init_kvcache(12, 5)
+    for row in dec2.workers:
+        for w in row:
+            w.migrate_blocks = (lambda w: lambda *a: setattr(w, "latest_migrate_event", FakeEvent(w.worker_id)))(w)
+    req = create_request(20, 21)
+    ctx.block_manager.allocate_blocks(req)
+    dec2._migrate_blocks(ctx.on_prefill_finished(req))
+    assert seen == [(21, [0, 1, 2, 3])]                     # every rank's copy waited for, then one call
+
+
+def test_requests_of_a_second_context_instance_carry_its_id_to_every_worker(engines):
+    ctx, dec = engines
+    model, cache = ctx.model_config, ctx.cache_config
+    calls = []
+
+    class InstanceWorker(FakeWorker):
+        def register_kvcache_mem_handles(self, ctx_pc, handles, context_instance=0):
+            calls.append(("register", context_instance))
+
+        def migrate_blocks(self, ctx_idx, ctx_pc, dec_idx, context_instance=0):
+            calls.append(("migrate", context_instance, list(ctx_idx)))
+
+    other = ContextStageLLMEngine(model, ParallelConfig(2, 0, 2, 0), cache, worker_factory=FakeWorker, instance_id=4)
+    other._init_kvcache(10, 0)
+    dec2 = DecodingStageLLMEngine(model, ParallelConfig(2, 0, 1, 0), cache, worker_factory=InstanceWorker)
+    dec2._init_kvcache(12, 0)
+    dec2.register_kvcache_mem_handles(ctx.parallel_config, ctx.kv_cache_mem_handles)
+    dec2.register_kvcache_mem_handles(other.parallel_config, other.kv_cache_mem_handles, context_instance=4)
+    assert calls == [("register", 0)] * 2 + [("register", 4)] * 2
+    calls.clear()
+    a, b = create_request(20, 31), create_request(20, 32)
+    ctx.block_manager.allocate_blocks(create_request(16, 30))
+    ctx.block_manager.allocate_blocks(a)
+    other.block_manager.allocate_blocks(b)
+    ma, mb = ctx.on_prefill_finished(a), other.on_prefill_finished(b)
+    assert (ma.context_instance, mb.context_instance) == (0, 4)
+    dec2._migrate_blocks(ma)
+    dec2._migrate_blocks(mb)
+    assert calls == [("migrate", 0, [1, 2])] * 2 + [("migrate", 4, [0, 1])] * 2
+    with pytest.raises(AssertionError, match="one context instance"):
+        dec2._migrate_blocks_batched([ctx.on_prefill_finished(a), mb])
