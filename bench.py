@@ -27,6 +27,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0   # MI355X published HBM3E bandwidth
+INFINITY_CACHE_BYTES = 256 << 20   # MI355X last-level cache in front of HBM
 
 
 def parse_args():
@@ -34,7 +35,12 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--config", type=int, default=2, choices=[1, 2, 3, 4, 5])
+    ap.add_argument("--config", type=int, default=0, choices=[0, 1, 2, 3, 4, 5],
+                    help="one configuration only (its full record, nothing else launched); default 0: configuration 2 "
+                         "as the headline and every other configuration after it, in one line")
+    ap.add_argument("--ctx-tp", type=int, default=0,
+                    help="configuration 4 only: context tensor-parallel size. 2 is the configuration itself (8 KiB runs "
+                         "at a 16 KiB source stride); 4 moves the same bytes from dense source pools, for comparison")
     ap.add_argument("--pattern", default="request", choices=["request", "batch", "handoff", "handoff-batched"],
                     help="handoff*: the same requests through Worker / BlockManager / the migration handoff "
                          "(torch ops, block allocation and release included), one call per request or one per batch")
@@ -55,25 +61,47 @@ def parse_args():
 
 
 def measured_traffic(config: int, algorithmic_bytes_per_launch: float):
-    """HBM bytes per launch from the committed hardware-counter summary of this configuration
-    (two rocprofv3 --pmc runs, FETCH_SIZE and WRITE_SIZE, each scaled by a plain copy of
-    known size), or None when no summary has been committed for it."""
+    """(HBM bytes per launch, where the figure comes from).  Hardware counters cannot be read
+    inside this run: the ratio of counted to algorithmic bytes is taken from the committed
+    counter summary of this configuration's kernel (two rocprofv3 --pmc runs, FETCH_SIZE and
+    WRITE_SIZE, each scaled by a plain copy of known size) and applied to this run's
+    algorithmic bytes.  (None, None) when no summary has been committed for it."""
     import re
 
-    path = os.path.join(ROOT, "profiles", f"kvm_copy_kernel_cfg{config}_pmc.txt")
+    name = f"profiles/kvm_copy_kernel_cfg{config}_pmc.txt"
+    path = os.path.join(ROOT, name)
     if not os.path.exists(path):
-        return None
+        return None, None
     m = re.search(r"TRAFFIC_PER_ALGORITHMIC_BYTE read=([0-9.]+) write=([0-9.]+)", open(path).read())
     if not m:
-        return None
+        return None, None
     # algorithmic bytes are half reads and half writes
-    return round(algorithmic_bytes_per_launch * (float(m.group(1)) + float(m.group(2))) / 2)
+    ratio = (float(m.group(1)) + float(m.group(2))) / 2
+    return round(algorithmic_bytes_per_launch * ratio), (
+        f"{name}: counted / algorithmic bytes = {ratio:.5f}, from the committed rocprofv3 counter runs of this "
+        "kernel, not from this run")
 
 
 def make_calls(w, pattern):
-    if pattern == "request" or w.recycles_blocks:
+    """Index lists of the calls of one step.  "request": one call per request.  "batch": one
+    call for everything; where the requests recycle block ids (configuration 4) that is not
+    possible, and consecutive requests are merged for as long as no block id, on either
+    side, occurs twice in the call -- what a decoding scheduler that batches its accepted
+    requests can do between two releases of context blocks."""
+    if pattern == "request":
         return [(c.ctx_idx, c.dec_idx) for c in w.calls]
-    return [([b for c in w.calls for b in c.ctx_idx], [b for c in w.calls for b in c.dec_idx])]
+    if not w.recycles_blocks:
+        return [([b for c in w.calls for b in c.ctx_idx], [b for c in w.calls for b in c.dec_idx])]
+    groups, ctx_seen, dec_seen = [], set(), set()
+    for c in w.calls:
+        if not groups or ctx_seen & set(c.ctx_idx) or dec_seen & set(c.dec_idx):
+            groups.append(([], []))
+            ctx_seen, dec_seen = set(), set()
+        groups[-1][0].extend(c.ctx_idx)
+        groups[-1][1].extend(c.dec_idx)
+        ctx_seen |= set(c.ctx_idx)
+        dec_seen |= set(c.dec_idx)
+    return groups
 
 
 def cpu_baseline(w, budget_s=12.0):
@@ -137,42 +165,42 @@ def cpu_baseline(w, budget_s=12.0):
     }
 
 
-def main():
-    args = parse_args()
-    if args.gpus != 1:
-        print("bench.py: this build measures one GPU only (source and destination pools share one HBM; "
-              "there is no sharding or collective on this path); run with --gpus 1", file=sys.stderr)
-        sys.exit(2)
+def load_workload(config: int, ctx_tp=None):
+    from distserve_amd import workloads
 
+    if config == 4 and ctx_tp:
+        return workloads.config4(ctx_tp=ctx_tp)
+    return {1: workloads.config1, 2: workloads.config2, 3: workloads.config3, 4: workloads.config4}[config]()
+
+
+def host_call_cost_us(cabi, geom, w, dst_k, dst_v, stream, calls=64):
+    """Host time of one kvm_migrate call with nothing queued behind it: one-block calls, each
+    issued on an idle stream and timed up to its return (validation, argument build and the
+    launch), the GPU drained before the next.  Median and best of `calls`."""
     import torch
 
-    if not torch.cuda.is_available():
-        print("bench.py: no GPU visible; the KV movement path has no CPU fallback", file=sys.stderr)
-        sys.exit(3)
+    first = w.calls[0]
+    ci, di = cabi.index_array(first.ctx_idx[:1]), cabi.index_array(first.dec_idx[:1])
+    costs = []
+    for _ in range(calls + 8):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        cabi.migrate(geom, ci, di, dst_k.data_ptr(), dst_v.data_ptr(), w.dst_blocks, stream.cuda_stream)
+        costs.append((time.perf_counter() - t0) * 1e6)
+    torch.cuda.synchronize()
+    costs = sorted(costs[8:])
+    return round(costs[len(costs) // 2], 2), round(costs[0], 2)
+
+
+def bench_migrate(config: int, pattern: str, steps: int, warmup: int, verify_result: bool = True,
+                  calibrate_copy: bool = False, ctx_tp=None):
+    """Times one migration workload; returns (record, workload).  Pools are made, timed and
+    freed inside."""
+    import torch
 
     from distserve_amd import cabi, workloads
 
-    for kv in args.opt:
-        name, value = kv.split("=")
-        cabi.set_option(name, int(value))
-
-    if args.plain_copy_only:
-        torch.cuda.set_device(0)
-        nbytes = args.plain_copy_only << 20
-        gbps = time_plain_copy(cabi, torch.cuda.current_stream(), nbytes=nbytes, reps=args.steps, warm=args.warmup)
-        print(json.dumps({"metric": "plain contiguous copy", "value": gbps, "unit": "GB/s",
-                          "bytes_copied_per_call": nbytes, "hbm_bytes_per_call": 2 * nbytes,
-                          "launches_per_call": -(-(nbytes // (8 << 20)) // 432), "steps": args.steps}))
-        return
-
-    if args.config == 5:
-        print(json.dumps(run_swap_bench(args)))
-        return
-
-    w = {1: workloads.config1, 2: workloads.config2, 3: workloads.config3, 4: workloads.config4}[args.config]()
-    if args.pattern.startswith("handoff"):
-        print(json.dumps(run_handoff_bench(args, w)))
-        return
+    w = load_workload(config, ctx_tp)
     torch.cuda.set_device(0)
     stream = torch.cuda.current_stream()
     s = w.shape
@@ -192,7 +220,7 @@ def main():
             cabi.register_source(w.ctx_pp, w.ctx_tp, p, t, s.num_layers, s.num_kv_heads,
                                  src_k[p][t].data_ptr(), src_v[p][t].data_ptr(),
                                  src_k[p][t].numel() * s.dtype_bytes)
-    calls = [(cabi.index_array(ci), cabi.index_array(di)) for ci, di in make_calls(w, args.pattern)]
+    calls = [(cabi.index_array(ci), cabi.index_array(di)) for ci, di in make_calls(w, pattern)]
     plan = cabi.migrate_plan(geom, max(len(c[0]) for c in calls), dst_k.data_ptr(), dst_v.data_ptr())
     launches_per_step = 0
     for ci, _ in calls:
@@ -202,91 +230,169 @@ def main():
         for ci, di in calls:
             cabi.migrate(geom, ci, di, dst_k.data_ptr(), dst_v.data_ptr(), w.dst_blocks, stream.cuda_stream)
 
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         step()
     torch.cuda.synchronize()
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    t_host0 = time.perf_counter()
     start.record(stream)
-    for _ in range(args.steps):
+    for _ in range(steps):
         step()
     stop.record(stream)
-    t_host_enqueued = time.perf_counter()
     torch.cuda.synchronize()
     elapsed_ms = start.elapsed_time(stop)
-    ms_per_step = elapsed_ms / args.steps
+    ms_per_step = elapsed_ms / steps
 
     # a second pass with an event between steps, for the spread (median and best step)
-    marks = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
     marks[0].record(stream)
-    for i in range(args.steps):
+    for i in range(steps):
         step()
         marks[i + 1].record(stream)
     torch.cuda.synchronize()
-    per_step_ms = sorted(marks[i].elapsed_time(marks[i + 1]) for i in range(args.steps))
+    per_step_ms = sorted(marks[i].elapsed_time(marks[i + 1]) for i in range(steps))
 
     payload = w.payload_bytes                       # bytes the decoding rank receives per step
     hbm_bytes = 2 * payload                         # each byte read once and written once
     hbm_gbps = hbm_bytes / (ms_per_step * 1e-3) / 1e9
-    launch_us = elapsed_ms * 1e3 / (args.steps * launches_per_step)
+    launch_us = elapsed_ms * 1e3 / (steps * launches_per_step)
     bytes_per_launch = hbm_bytes / launches_per_step
 
-    bit_exact = None
-    if not args.no_verify:
-        bit_exact = verify(w, src_k, src_v, dst_k, dst_v)
+    bit_exact = verify(w, src_k, src_v, dst_k, dst_v) if verify_result else None
+    host_call_us, host_call_us_min = host_call_cost_us(cabi, geom, w, dst_k, dst_v, stream)
+    copy_ceiling = time_plain_copy(cabi, stream) if calibrate_copy else None
 
-    copy_ceiling = None
-    if args.calibrate_copy:
-        copy_ceiling = time_plain_copy(cabi, stream)
-
+    tuning = {k: cabi.get_option(k) for k in ("tile_bytes", "threads", "unroll", "nt_load", "nt_store")}
+    traffic, traffic_source = measured_traffic(config if not ctx_tp else 0, bytes_per_launch)
+    cache_resident = 2 * hbm_bytes <= INFINITY_CACHE_BYTES
     out = {
-        "metric": "KV migration GB/s (% of HBM peak) + us/request at LLaMA-2-7B shape" if args.config == 2
+        "metric": "KV migration GB/s (% of HBM peak) + us/request at LLaMA-2-7B shape" if config == 2
                   else f"KV migration GB/s (% of HBM peak) + us/request, {w.name}",
         "value": round(hbm_gbps, 2), "unit": "GB/s",
-        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u8", "data": "synthetic",
         "config": {
             "workload": (f"{w.name}: {len(w.calls)} requests, {w.total_blocks} blocks of "
                          f"{w.payload_bytes_per_block} B (K+V, decoding rank's share), context pp{w.ctx_pp}/tp{w.ctx_tp}"
                          f" -> decoding pp{w.dec_pp}/tp{w.dec_tp} rank ({w.dec_pp_rank},{w.dec_tp_rank}), "
                          f"pools {w.src_blocks}/{w.dst_blocks} blocks, seed {w.seed}"),
-            "pattern": "one call per request" if len(calls) > 1 else "one call per batch",
+            "pattern": ("one call per request" if pattern == "request" else
+                        f"{len(calls)} calls per batch (requests merged until a block id recurs)" if len(calls) > 1
+                        else "one call per batch"),
             "value_counts": "HBM bytes read + written (2 x payload) per second",
-            "tuning": {k: cabi.get_option(k) for k in ("tile_bytes", "threads", "unroll", "nt_load", "nt_store")},
+            "tuning": tuning,
         },
         "ms_per_step_median": round(per_step_ms[len(per_step_ms) // 2], 4), "ms_per_step_min": round(per_step_ms[0], 4),
         "payload_GBps": round(payload / (ms_per_step * 1e-3) / 1e9, 2),
         "frac_of_hbm_peak": round(hbm_gbps / HBM_PEAK_GBPS, 4),
         "us_per_request": round(ms_per_step * 1e3 / len(w.calls), 2),
         "blocks_per_s": round(w.total_blocks / (ms_per_step * 1e-3), 1),
-        "host_enqueue_us_per_call": round((t_host_enqueued - t_host0) * 1e6 / (args.steps * len(calls)), 2),
+        "host_call_us": host_call_us, "host_call_us_min": host_call_us_min,
         "bit_exact": bit_exact,
         "roofline": {
             "bound": "hbm", "achieved": round(bytes_per_launch / (launch_us * 1e-6) / 1e9, 2), "peak": HBM_PEAK_GBPS,
             "unit": "GB/s", "frac": round(bytes_per_launch / (launch_us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
-            "traffic": measured_traffic(args.config, bytes_per_launch),
-            "kernel": ("kvm_copy_simple_kernel" if plan["simple_kernel"] else "kvm_copy_kernel") + "<u32x4, 64, 1>",
+            "traffic": traffic, "traffic_source": traffic_source,
+            "kernel": (("kvm_copy_simple_kernel" if plan["simple_kernel"] else "kvm_copy_kernel")
+                       + f"<u32x{plan['vector_bytes'] // 4}, {plan['threads']}, {cabi.get_option('unroll')}>"),
             "launches_per_step": launches_per_step,
             "avg_launch_us": round(launch_us, 2), "algorithmic_bytes_per_launch": round(bytes_per_launch),
             "workgroups_per_block": plan["workgroups_per_block"], "workgroup_size": plan["threads"],
         },
     }
+    if cache_resident:
+        # a step's reads and writes fit the 256 MB last-level cache and the steps repeat them:
+        # the figure is a cache and launch-latency figure, not an HBM one
+        out["cache_resident"] = True
     if copy_ceiling is not None:
         out["plain_copy_GBps"] = copy_ceiling
+    del src_k, src_v, dst_k, dst_v
+    cabi.reset()
+    torch.cuda.empty_cache()
+    return out, w
+
+
+def compact(d: dict) -> dict:
+    """The figures of one configuration as they ride along in the headline line."""
+    keys = ("value", "frac_of_hbm_peak", "us_per_request", "blocks_per_s", "payload_GBps", "ms_per_step",
+            "host_call_us", "bit_exact", "cache_resident")
+    out = {("GBps" if k == "value" else "frac" if k == "frac_of_hbm_peak" else k): d[k] for k in keys if k in d}
+    out["pattern"] = d["config"]["pattern"]
+    out["launches_per_step"] = d["roofline"]["launches_per_step"]
+    out["avg_launch_us"] = d["roofline"]["avg_launch_us"]
+    out["kernel"] = d["roofline"]["kernel"]
+    return out
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (source and destination pools share one HBM; "
+              "there is no sharding or collective on this path); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the KV movement path has no CPU fallback", file=sys.stderr)
+        sys.exit(3)
+
+    from distserve_amd import cabi
+
+    for kv in args.opt:
+        name, value = kv.split("=")
+        cabi.set_option(name, int(value))
+
+    if args.plain_copy_only:
+        torch.cuda.set_device(0)
+        nbytes = args.plain_copy_only << 20
+        gbps = time_plain_copy(cabi, torch.cuda.current_stream(), nbytes=nbytes, reps=args.steps, warm=args.warmup)
+        print(json.dumps({"metric": "plain contiguous copy", "value": gbps, "unit": "GB/s",
+                          "bytes_copied_per_call": nbytes, "hbm_bytes_per_call": 2 * nbytes,
+                          "launches_per_call": -(-(nbytes // (8 << 20)) // 432), "steps": args.steps}))
+        return
+
+    if args.config == 5:
+        print(json.dumps(run_swap_bench(args)))
+        return
+
+    if args.pattern.startswith("handoff"):
+        print(json.dumps(run_handoff_bench(args, load_workload(args.config or 2))))
+        return
+
+    verify_result = not args.no_verify
+    if args.config:
+        # one configuration, nothing else launched: the command the kernel profiles are taken with
+        out, w = bench_migrate(args.config, args.pattern, args.steps, args.warmup, verify_result,
+                               args.calibrate_copy, args.ctx_tp)
+        if not args.no_cpu_baseline:
+            out["cpu_baseline"] = cpu_baseline(w)
+        print(json.dumps(out))
+        return
+
+    # The default run: configuration 2, one call per request, is the headline; every other
+    # configuration follows in its own pools and rides along in "configs".
+    out, w2 = bench_migrate(2, "request", args.steps, args.warmup, verify_result, args.calibrate_copy)
+    configs = {}
+    for cfg, pattern in ((2, "batch"), (1, "request"), (3, "request"), (3, "batch"), (4, "request"), (4, "batch")):
+        d, _ = bench_migrate(cfg, pattern, args.steps, args.warmup, verify_result)
+        key = f"cfg{cfg}" if pattern == "request" else f"cfg{cfg}_batched"
+        configs[key] = compact(d)
+    swap = run_swap_bench(args, default_only=True)
+    configs["cfg5"] = swap
+    out["configs"] = configs
     if not args.no_cpu_baseline:
-        del src_k, src_v, dst_k, dst_v
-        torch.cuda.empty_cache()
-        out["cpu_baseline"] = cpu_baseline(w)
+        out["cpu_baseline"] = cpu_baseline(w2)
     print(json.dumps(out))
 
 
-def run_swap_bench(args):
+def run_swap_bench(args, default_only: bool = False):
     """Configuration 5: swap 2048 blocks (16 GiB) from HBM to a pinned host pool and back into
     other GPU slots, on side streams, while an 8-request migration runs on the main stream.
     The denominator is the host link measured in the same run with one large pinned copy per
     direction.  A step is one swap-out plus one swap-in of the whole block list.  Every
     implementation is timed three times: alone, beside the 8-request migration (the headline
-    row), and beside migrations issued back to back for as long as both swaps take."""
+    row), and beside migrations issued back to back for as long as both swaps take.
+    ``default_only``: only the implementation the library's default takes, reported compactly."""
     import torch
 
     from distserve_amd import cabi, workloads
@@ -356,13 +462,14 @@ def run_swap_bench(args):
 
     results = {}
     bytes_dir = w.bytes_per_direction
-    option_mode, default_wgs = cabi.get_option("swap_mode"), cabi.get_option("swap_wgs")
-    if args.swap_wgs is None:
-        args.swap_wgs = [default_wgs]
+    option_mode = cabi.get_option("swap_mode")
+    default_wgs = (cabi.get_option("swap_wgs"), cabi.get_option("swap_wgs_in"))     # swap-out, swap-in
+    # --swap-wgs N gives both directions N workgroups; the library's own pair is always measured
+    wgs_list = [(g, g) for g in (args.swap_wgs or [])]
     # what the library's default takes for this block list (mode 3 decides per call)
     default_mode = cabi.swap_plan(w.out_gpu_ids, w.out_host_ids, slab)["mode"]
-    if default_mode == 1 and default_wgs not in args.swap_wgs:
-        args.swap_wgs.append(default_wgs)
+    if default_mode == 1 and default_wgs not in wgs_list:
+        wgs_list.append(default_wgs)
 
     def migrate_timed():
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -382,11 +489,15 @@ def run_swap_bench(args):
     migrate_alone_ms = e0.elapsed_time(e1)
 
     variants = [("hipMemcpyAsync per block", 0, None), ("hipMemcpyAsync per block, V on a forked stream", 2, None)]
-    variants += [(f"copy kernel over pinned memory, {g} workgroups per pool kind", 1, g) for g in args.swap_wgs]
+    variants += [(f"copy kernel over pinned memory, {g[0]} (out) / {g[1]} (in) workgroups per pool kind", 1, g)
+                 for g in wgs_list]
+    if default_only:
+        variants = [v for v in variants if v[1] == default_mode and (v[2] is None or v[2] == default_wgs)]
     for mode_name, mode, wgs in variants:
         cabi.set_option("swap_mode", mode)
         if wgs:
-            cabi.set_option("swap_wgs", wgs)
+            cabi.set_option("swap_wgs", wgs[0])
+            cabi.set_option("swap_wgs_in", wgs[1])
         rows = []
         for phase in ("alone", "overlapped", "busy"):
             overlapped = phase != "alone"
@@ -452,15 +563,39 @@ def run_swap_bench(args):
             rows.append(row)
         results[mode_name] = rows
     cabi.set_option("swap_mode", option_mode)
-    cabi.set_option("swap_wgs", default_wgs)
+    cabi.set_option("swap_wgs", default_wgs[0])
+    cabi.set_option("swap_wgs_in", default_wgs[1])
     cpu = None
-    if not args.no_cpu_baseline:
+    if not args.no_cpu_baseline and not default_only:
         del k_ref, v_ref, src_k, src_v
         cpu = swap_cpu_baseline(w)
     default_name = [n for n, m, g in variants if m == default_mode and (g is None or g == default_wgs)]
     best = results[default_name[0] if default_name else variants[0][0]][1]
     total_s = best["swap_out_ms"] * 1e-3 + best["swap_in_ms"] * 1e-3
     cabi.reset()
+    if default_only:
+        alone, beside, busy = results[default_name[0]]
+        pick = ("swap_out_frac_of_link", "swap_in_frac_of_link", "swap_out_GBps", "swap_in_GBps")
+        return {
+            "workload": (f"{w.name}: {len(w.out_gpu_ids)} blocks x {2 * slab} B (K+V) out to a pinned pool and back "
+                         f"into other slots, beside a migration of {len(mig.calls)} requests on another stream"),
+            "swap_implementation": default_name[0],
+            "GBps": round(2 * bytes_dir / total_s / 1e9, 2),
+            "link_GBps": {k: round(v, 2) for k, v in link.items()},
+            "frac_of_link": round(2 * bytes_dir / total_s / 1e9 / ((link["d2h"] + link["h2d"]) / 2), 4),
+            "alone": {k: alone[k] for k in pick},
+            "beside_8_requests": {k: beside[k] for k in pick},
+            "beside_continuous_migration": {k: busy[k] for k in pick},
+            "host_enqueue_us": {"swap_out_alone": alone["host_enqueue_swap_out_us"],
+                                "swap_out_beside_8_requests": beside["host_enqueue_swap_out_us"]},
+            "migration_ms": {"alone": beside["migration_ms_alone"],
+                             "beside_swap_out": beside["migration_ms_beside_swap_out"],
+                             "beside_swap_in": beside["migration_ms_beside_swap_in"],
+                             "continuous_avg": busy["migration_ms_avg_of_continuous"]},
+            "blocks_per_s": round(2 * len(w.out_gpu_ids) / total_s, 1),
+            "bit_exact": bool(alone["round_trip_bit_exact"] and beside["round_trip_bit_exact"]
+                              and busy["round_trip_bit_exact"]),
+        }
     return {
         "metric": ("KV swap GB/s (fraction of measured host link), "
                    + (f"pools of {args.swap_shape} layers,heads,head_dim" if args.swap_shape else "LLaMA-2-7B shape")
@@ -584,6 +719,19 @@ def run_handoff_bench(args, w):
         h, t, tables = one_step(args.warmup + i)
         host_s += h
         total_s += t
+    # "Transmission" as the reference's plots derive it from the lifetime events
+    # (migration_end - migration_begin): once as the reference stamps it, when the asynchronous
+    # calls have returned, and once with the end stamped after the copy has finished on the GPU
+    from distserve_amd.lifetime import transmission_seconds
+
+    transmission_us = {}
+    for name, wait in (("stamped_at_enqueue", False), ("stamped_after_the_copy", True)):
+        dec.gpu_complete_lifetime_events = wait
+        dec.lifetime_events.clear()
+        one_step(args.warmup + args.steps + (1 if wait else 0))
+        spans = [transmission_seconds(ev) for ev in dec.lifetime_events.values()]
+        transmission_us[name] = round(sum(spans) / len(spans) * 1e6, 2)
+    dec.gpu_complete_lifetime_events = False
     # the tables the BlockManagers produced are the workload's own
     same_tables = all(ci == c.ctx_idx and di == c.dec_idx for (ci, di), c in zip(tables, w.calls))
     dw = dec.workers[0][0]
@@ -603,6 +751,10 @@ def run_handoff_bench(args, w):
                    "value_counts": "HBM bytes read + written per second of host wall clock (allocation to GPU idle)"},
         "us_per_request": round(ms_per_step * 1e3 / len(w.calls), 2),
         "host_us_per_request": round(host_s / args.steps / len(w.calls) * 1e6, 2),
+        "transmission_us_per_request": transmission_us["stamped_after_the_copy"],
+        "transmission_us_per_request_stamped_at_enqueue": transmission_us["stamped_at_enqueue"],
+        "transmission_note": ("mean of migration_end - migration_begin over the requests of one step, as the reference's "
+                              "plots compute it; batched: every request of the call spans the whole call"),
         "frac_of_hbm_peak": round(hbm_gbps / HBM_PEAK_GBPS, 4),
         "block_tables_equal_workload": same_tables, "bit_exact": bit_exact,
     }

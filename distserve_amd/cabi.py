@@ -72,7 +72,7 @@ def _load() -> ctypes.CDLL:
     lib.kvm_get_option.argtypes = [ctypes.c_char_p]
     lib.kvm_get_option.restype = i64
     lib.kvm_migrate_plan.argtypes = [ctypes.POINTER(KvmGeom), i64, vp, vp, ip]
-    lib.kvm_swap_plan.argtypes = [ip, ip, i64, i64, ip]
+    lib.kvm_swap_plan.argtypes = [ip, ip, i64, i64, ctypes.c_int, ip]
     lib.kvm_debug_divide.argtypes = [ctypes.c_uint32, ctypes.c_uint32]
     lib.kvm_debug_divide.restype = ctypes.c_uint32
     for name in EXPORTS:
@@ -176,11 +176,11 @@ def get_option(name: str) -> int:
     return v
 
 
-def swap_plan(src_ids: Sequence[int], dst_ids: Sequence[int], slab_bytes: int) -> dict:
+def swap_plan(src_ids: Sequence[int], dst_ids: Sequence[int], slab_bytes: int, is_swap_in: bool = False) -> dict:
     if len(src_ids) != len(dst_ids):
         raise KvmError(KVM_EINVAL, f"{len(src_ids)} source blocks but {len(dst_ids)} target blocks")
     out = (ctypes.c_int64 * 4)()
-    _check(lib.kvm_swap_plan(_arr(src_ids), _arr(dst_ids), len(src_ids), slab_bytes, out))
+    _check(lib.kvm_swap_plan(_arr(src_ids), _arr(dst_ids), len(src_ids), slab_bytes, 1 if is_swap_in else 0, out))
     return dict(zip(("mode", "copies_per_pool", "launches", "workgroups_per_pool_kind"), list(out)))
 
 

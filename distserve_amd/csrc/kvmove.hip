@@ -380,7 +380,8 @@ std::atomic<int64_t> opt_nt_load{1};
 std::atomic<int64_t> opt_nt_store{1};
 std::atomic<int64_t> opt_swap_mode{3};
 std::atomic<int64_t> opt_swap_wgs{8};
-std::atomic<int64_t> opt_swap_kernel_below{2 << 20};
+std::atomic<int64_t> opt_swap_wgs_in{10};
+std::atomic<int64_t> opt_swap_kernel_below{1ll << 32};
 std::atomic<int64_t> opt_lds_pad{0};
 std::atomic<int64_t> opt_wave_contig{0};
 std::atomic<int64_t> opt_xcd_map{1};
@@ -396,6 +397,7 @@ std::atomic<int64_t> *find_opt(const char *name)
     if (!strcmp(name, "nt_store")) return &opt_nt_store;
     if (!strcmp(name, "swap_mode")) return &opt_swap_mode;
     if (!strcmp(name, "swap_wgs")) return &opt_swap_wgs;
+    if (!strcmp(name, "swap_wgs_in")) return &opt_swap_wgs_in;
     if (!strcmp(name, "swap_kernel_below")) return &opt_swap_kernel_below;
     if (!strcmp(name, "lds_pad")) return &opt_lds_pad;
     if (!strcmp(name, "wave_contig")) return &opt_wave_contig;
@@ -925,9 +927,11 @@ int get_fork(bool is_swap_in, Fork **out)
 }
 
 // Which implementation serves a swap call (0, 1 or 2; see the "swap_mode" option).  Mode 3
-// decides per call: a copy engine needs about 2 MiB per copy to hide its per-copy cost
-// (measured: 4 MiB copies reach 98 % of the link, 1 MiB 85-91 %, 288 KiB 55 %, 64 KiB 20 %),
-// the copy kernel does not care (90-99 % at every slab size).  *out_runs = copies per pool.
+// takes the copy kernel unless the call's copies average "swap_kernel_below" bytes or more: the
+// kernel fills 97-100 % of the link at every slab size for a tenth of a millisecond of host
+// time per call, where the copy engines need 2 MiB and more per copy to hide their per-copy
+// cost (4 MiB copies 98 % of the link, 1 MiB 85-91 %, 288 KiB 55 %, 64 KiB 20 %) and two
+// runtime calls per block (4-5 ms for 2048 blocks).  *out_runs = copies per pool.
 int64_t swap_mode_for(const IdxPair *pairs, int64_t n, int64_t slab_bytes, int64_t *out_runs)
 {
     int64_t runs = n > 0 ? 1 : 0;
@@ -957,7 +961,7 @@ int kvm_set_option(const char *name, int64_t value)
     if (o == &opt_tile_bytes) ok = value == 0 || (value >= 1024 && value <= (1 << 26) && (value & (value - 1)) == 0);
     else if (o == &opt_threads) ok = value == 64 || value == 128 || value == 256 || value == 512 || value == 1024;
     else if (o == &opt_unroll) ok = value == 1 || value == 2 || value == 4 || value == 8 || value == 16;
-    else if (o == &opt_swap_wgs) ok = value >= 1 && value <= 4096;
+    else if (o == &opt_swap_wgs || o == &opt_swap_wgs_in) ok = value >= 1 && value <= 4096;
     else if (o == &opt_lds_pad) ok = value >= 0 && value <= 65536;
     else if (o == &opt_xcd_map) ok = value >= 0 && value <= 3;
     else if (o == &opt_swap_mode) ok = value >= 0 && value <= 3;
@@ -1234,7 +1238,8 @@ int kvm_migrate(const KvmGeom *geom, const int64_t *ctx_idx, const int64_t *dec_
                        plan.dst_block_stride, plan.vec, (hipStream_t)stream, nullptr, nullptr, nullptr);
 }
 
-int kvm_swap_plan(const int64_t *src_ids, const int64_t *dst_ids, int64_t n, int64_t slab_bytes, int64_t out[4])
+int kvm_swap_plan(const int64_t *src_ids, const int64_t *dst_ids, int64_t n, int64_t slab_bytes, int is_swap_in,
+                  int64_t out[4])
 {
     if (!out) return fail(KVM_EINVAL, "out is null");
     if (n < 0 || (n > 0 && (!src_ids || !dst_ids))) return fail(KVM_EINVAL, "bad index lists");
@@ -1251,7 +1256,7 @@ int kvm_swap_plan(const int64_t *src_ids, const int64_t *dst_ids, int64_t n, int
     out[0] = mode;
     out[1] = runs;
     out[2] = mode == 1 ? (n + kMaxIdx - 1) / kMaxIdx : 0;
-    out[3] = mode == 1 ? opt_swap_wgs.load() : 0;
+    out[3] = mode == 1 ? (is_swap_in ? opt_swap_wgs_in.load() : opt_swap_wgs.load()) : 0;
     return KVM_OK;
 }
 
@@ -1313,7 +1318,7 @@ int kvm_swap(const int64_t *src_ids, const int64_t *dst_ids, int64_t n, int is_s
         const int vec = vec_width((uint64_t)slab_bytes | (uintptr_t)src_k | (uintptr_t)src_v |
                                   (uintptr_t)dst_k | (uintptr_t)dst_v);
         return launch_copy({s}, pairs.data(), n, dst_k, dst_v, (uint64_t)slab_bytes, vec, st, nullptr,
-                           nullptr, nullptr, (int)opt_swap_wgs.load());
+                           nullptr, nullptr, (int)(is_swap_in ? opt_swap_wgs_in.load() : opt_swap_wgs.load()));
     }
 
     // hipMemcpyAsync per run of blocks that are consecutive on both sides.  In mode 2 the V

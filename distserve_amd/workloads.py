@@ -171,13 +171,16 @@ def config3(seed: int = 3, num_requests: int = 32) -> MigrateWorkload:
     return w
 
 
-def config4(seed: int = 4, num_requests: int = 24) -> MigrateWorkload:
+def config4(seed: int = 4, num_requests: int = 24, ctx_tp: int = 2) -> MigrateWorkload:
     """LLaMA-2-70B GQA KV shape, context TP2/PP2 -> decoding TP4 rank 1 (2 of 8 KV heads,
     all 80 layers).  The batch needs more blocks than either pool holds, so the calls
-    recycle block ids."""
+    recycle block ids.  ``ctx_tp=4`` is a comparison layout, not the configuration: the same
+    block tables and the same bytes, from context pools that hold exactly the two heads
+    the decoding rank wants, so the sources are read densely."""
     g = torch.Generator().manual_seed(seed)
     shape = KvShape(80, 8, 128)
-    w = MigrateWorkload("cfg4-llama2-70b-tp2pp2to-tp4r1", shape, 2, 2, 1, 4, 0, 1, 1024, 2048, seed,
+    name = "cfg4-llama2-70b-tp2pp2to-tp4r1" if ctx_tp == 2 else f"cfg4-variant-tp{ctx_tp}pp2to-tp4r1"
+    w = MigrateWorkload(name, shape, 2, ctx_tp, 1, 4, 0, 1, 1024, 2048, seed,
                         recycles_blocks=True)
     w.calls = _recycled_calls(g, _lengths(g, num_requests, 256, 4096), 16, 1024, 2048)
     return w

@@ -173,19 +173,24 @@ int kvm_copy_plain(void *dst, const void *src, int64_t nbytes, void *stream);
  *                    reports KVM_EINVAL for one that is not)
  *   "nt_load"        1 = nontemporal loads, 0 = plain
  *   "nt_store"       1 = nontemporal stores, 0 = plain
- *   "swap_mode"      3 (default) = chosen per call: mode 2 when the copies of the call average
- *                        at least "swap_kernel_below" bytes each, else mode 1,
+ *   "swap_mode"      3 (default) = chosen per call: mode 1, unless the copies of the call average
+ *                        "swap_kernel_below" bytes or more each or the pinned pools are not mapped
+ *                        for device access, then mode 2,
+ *                    1 = copy kernel that reads/writes the pinned pools in place: one launch
+ *                        per 432 blocks whatever their size, about 0.1 ms of host time for 2048
+ *                        blocks, 97-100 % of the link,
  *                    2 = hipMemcpyAsync per run of blocks consecutive on both sides, K pool on
  *                        the caller's stream and V pool on a second stream forked from and
- *                        joined back into it,
- *                    0 = the same with both pools on the caller's stream,
- *                    1 = copy kernel that reads/writes the pinned pools in place: one launch
- *                        per 432 blocks whatever their size, a few microseconds of host time
- *   "swap_wgs"       workgroups per pool kind of the swap kernel, 1..4096.  Default 8: 99 % of
- *                    the link on an idle GPU and 87-96 % while other kernels saturate HBM;
- *                    10-12 hold 96-98 % under such load but slow short kernels beside them,
- *                    32 and more slow every HBM-bound kernel several times over
- *   "swap_kernel_below"  bytes per copy under which mode 3 takes the kernel (default 2 MiB)
+ *                        joined back into it: two runtime calls per block (4-5 ms of host time
+ *                        for 2048 blocks), 97-98 % of the link for copies of 4 MiB, less below,
+ *                    0 = the same with both pools on the caller's stream (87 %)
+ *   "swap_wgs"       workgroups per pool kind of the swap kernel for a swap-out, 1..4096.  Default 8:
+ *                    99 % of the link on an idle GPU and 96 % while other kernels saturate HBM
+ *   "swap_wgs_in"    the same for a swap-in.  Default 10: 98 % idle, 98 % beside kernels that
+ *                    saturate HBM, where 8 workgroups fall to 86 %; more workgroups slow the
+ *                    kernels beside the swap (12: +5 %, 16: +20 %, 32: several times)
+ *   "swap_kernel_below"  bytes per copy under which mode 3 takes the kernel (default 4 GiB, i.e.
+ *                    always; 2 MiB hands large slabs to the copy engines)
  * kvm_get_option returns the value or KVM_EINVAL (as int64) for an unknown name.
  */
 int kvm_set_option(const char *name, int64_t value);
@@ -211,10 +216,11 @@ int kvm_migrate_plan(const KvmGeom *geom, int64_t n, const void *dst_k, const vo
  * tests and reports (no counterpart in the reference): out[0] = implementation taken (0, 1
  * or 2, as "swap_mode" numbers them), out[1] = copies per pool = runs of blocks consecutive
  * on both sides, out[2] = kernel launches (mode 1, else 0), out[3] = workgroups per pool
- * kind of each launch (mode 1, else 0).  Touches no device and no pool.
+ * kind of each launch (mode 1, else 0; swap-in and swap-out have their own counts).  Touches
+ * no device and no pool (so it cannot see whether pinned pools are mapped for the kernel).
  */
 int kvm_swap_plan(const int64_t *src_ids, const int64_t *dst_ids, int64_t n, int64_t slab_bytes,
-                  int64_t out[4]);
+                  int is_swap_in, int64_t out[4]);
 
 /*
  * Test hook (no counterpart in the reference): n / d computed the way the kernel computes

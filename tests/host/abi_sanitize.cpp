@@ -39,7 +39,7 @@ int main()
     EXPECT(std::strlen(kvm_last_error()) == 0);
 
     // options: every name, valid and invalid values, unknown and null names
-    const char *names[] = {"tile_bytes", "threads", "unroll", "nt_load", "nt_store", "swap_mode", "swap_wgs",
+    const char *names[] = {"tile_bytes", "threads", "unroll", "nt_load", "nt_store", "swap_mode", "swap_wgs", "swap_wgs_in",
                            "lds_pad", "wave_contig", "xcd_map", "simple"};
     for (const char *n : names) {
         const int64_t old = kvm_get_option(n);
@@ -182,10 +182,15 @@ int main()
 
     // the swap plan touches no device: run lists of many shapes through it
     int64_t sp[4];
-    EXPECT(kvm_swap_plan(ci.data(), di.data(), 1, 64, nullptr) == KVM_EINVAL);
-    EXPECT(kvm_swap_plan(nullptr, di.data(), 1, 64, sp) == KVM_EINVAL);
-    EXPECT(kvm_swap_plan(ci.data(), di.data(), 1, 0, sp) == KVM_EINVAL);
-    EXPECT(kvm_swap_plan(nullptr, nullptr, 0, 64, sp) == KVM_OK && sp[1] == 0);
+    EXPECT(kvm_swap_plan(ci.data(), di.data(), 1, 64, 0, nullptr) == KVM_EINVAL);
+    EXPECT(kvm_swap_plan(nullptr, di.data(), 1, 64, 0, sp) == KVM_EINVAL);
+    EXPECT(kvm_swap_plan(ci.data(), di.data(), 1, 0, 0, sp) == KVM_EINVAL);
+    EXPECT(kvm_swap_plan(nullptr, nullptr, 0, 64, 0, sp) == KVM_OK && sp[1] == 0);
+    // the default takes the copy kernel whatever the slab size, with its own workgroup count per direction
+    EXPECT(kvm_swap_plan(ci.data(), di.data(), 5, 4 << 20, 0, sp) == KVM_OK && sp[0] == 1 && sp[3] == kvm_get_option("swap_wgs"));
+    EXPECT(kvm_swap_plan(ci.data(), di.data(), 5, 4 << 20, 1, sp) == KVM_OK && sp[0] == 1 && sp[3] == kvm_get_option("swap_wgs_in"));
+    // with a threshold, large copies go to the copy engines as before
+    EXPECT(kvm_set_option("swap_kernel_below", 2 << 20) == KVM_OK);
     for (int round = 0; round < 200; ++round) {
         const int64_t n = (int64_t)(rng() % 3000);
         std::vector<int64_t> a((size_t)n), b((size_t)n);
@@ -197,13 +202,14 @@ int main()
             if (i > 0 && !(a[(size_t)i] == a[(size_t)i - 1] + 1 && b[(size_t)i] == b[(size_t)i - 1] + 1)) ++runs;
         }
         const int64_t slab = (int64_t)1 << (rng() % 24);
-        EXPECT(kvm_swap_plan(a.data(), b.data(), n, slab, sp) == KVM_OK);
+        EXPECT(kvm_swap_plan(a.data(), b.data(), n, slab, round & 1, sp) == KVM_OK);
         EXPECT(sp[1] == runs);
         const int64_t want = runs > 0 && n * slab / runs < (2 << 20) ? 1 : 2;
         EXPECT(sp[0] == want);
         EXPECT(sp[2] == (want == 1 ? (n + 431) / 432 : 0));
         if (failures) break;
     }
+    EXPECT(kvm_set_option("swap_kernel_below", 1ll << 32) == KVM_OK);
 
     // the divider arithmetic, many operands
     for (int i = 0; i < 200000; ++i) {

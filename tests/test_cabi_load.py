@@ -31,40 +31,46 @@ def test_version_and_options(kvm):
     assert kvm.get_option("unroll") == 8
     kvm.set_option("unroll", old)
     for name, bad in (("tile_bytes", 5000), ("threads", 100), ("unroll", 3), ("nt_store", 2), ("swap_mode", 4),
-                      ("swap_wgs", 0), ("swap_kernel_below", -1), ("nope", 1)):
+                      ("swap_wgs", 0), ("swap_wgs_in", 5000), ("swap_kernel_below", -1), ("nope", 1)):
         with pytest.raises(kvm.KvmError) as e:
             kvm.set_option(name, bad)
         assert e.value.code == kvm.KVM_EINVAL
 
 
-def test_swap_plan_picks_the_implementation_by_bytes_per_copy(kvm):
-    """Default mode: the copy kernel for copies under 2 MiB each, copy engines above; runs of
-    blocks consecutive on both sides count as one copy."""
-    assert kvm.get_option("swap_mode") == 3 and kvm.get_option("swap_kernel_below") == 2 << 20
+def test_swap_plan_takes_the_kernel_by_default_and_the_engines_above_a_threshold(kvm):
+    """Default: the copy kernel whatever the slab size, with its own workgroup count per
+    direction.  With a "swap_kernel_below" threshold, calls whose copies average that many
+    bytes go to the copy engines; runs of blocks consecutive on both sides count as one copy."""
+    assert kvm.get_option("swap_mode") == 3 and kvm.get_option("swap_kernel_below") == 1 << 32
+    assert kvm.get_option("swap_wgs") == 8 and kvm.get_option("swap_wgs_in") == 10
     scattered = ([5, 9, 2, 7], [1, 8, 3, 6])
-    assert kvm.swap_plan(*scattered, 4 << 20) == {"mode": 2, "copies_per_pool": 4, "launches": 0,
-                                                  "workgroups_per_pool_kind": 0}
-    assert kvm.swap_plan(*scattered, 2 << 20)["mode"] == 2
-    plan = kvm.swap_plan(*scattered, (2 << 20) - 16)
-    assert plan == {"mode": 1, "copies_per_pool": 4, "launches": 1,
-                    "workgroups_per_pool_kind": kvm.get_option("swap_wgs")}
-    # 8 consecutive blocks of 288 KiB are one 2.25 MiB copy; broken in two they are not
-    run = list(range(10, 18))
-    assert kvm.swap_plan(run, list(range(40, 48)), 288 << 10) == {"mode": 2, "copies_per_pool": 1, "launches": 0,
-                                                                   "workgroups_per_pool_kind": 0}
-    assert kvm.swap_plan(run, list(range(40, 44)) + list(range(50, 54)), 288 << 10)["mode"] == 1
-    assert kvm.swap_plan(run, run[::-1], 288 << 10)["copies_per_pool"] == 8
-    assert kvm.swap_plan(list(range(1000)), list(range(1000)), 4096)["mode"] == 2          # one 4 MiB run
-    assert kvm.swap_plan(list(range(0, 2000, 2)), list(range(1000)), 4096)["launches"] == 3  # 432 blocks per launch
+    assert kvm.swap_plan(*scattered, 4 << 20) == {"mode": 1, "copies_per_pool": 4, "launches": 1,
+                                                  "workgroups_per_pool_kind": 8}
+    assert kvm.swap_plan(*scattered, 4 << 20, is_swap_in=True)["workgroups_per_pool_kind"] == 10
+    assert kvm.swap_plan(list(range(0, 2000, 2)), list(range(1000)), 4096)["launches"] == 3   # 432 blocks per launch
     assert kvm.swap_plan([], [], 4096) == {"mode": 2, "copies_per_pool": 0, "launches": 0, "workgroups_per_pool_kind": 0}
+    kvm.set_option("swap_kernel_below", 2 << 20)
+    try:
+        assert kvm.swap_plan(*scattered, 4 << 20) == {"mode": 2, "copies_per_pool": 4, "launches": 0,
+                                                      "workgroups_per_pool_kind": 0}
+        assert kvm.swap_plan(*scattered, 2 << 20)["mode"] == 2
+        assert kvm.swap_plan(*scattered, (2 << 20) - 16)["mode"] == 1
+        # 8 consecutive blocks of 288 KiB are one 2.25 MiB copy; broken in two they are not
+        run = list(range(10, 18))
+        assert kvm.swap_plan(run, list(range(40, 48)), 288 << 10) == {"mode": 2, "copies_per_pool": 1, "launches": 0,
+                                                                       "workgroups_per_pool_kind": 0}
+        assert kvm.swap_plan(run, list(range(40, 44)) + list(range(50, 54)), 288 << 10)["mode"] == 1
+        assert kvm.swap_plan(run, run[::-1], 288 << 10)["copies_per_pool"] == 8
+        assert kvm.swap_plan(list(range(1000)), list(range(1000)), 4096)["mode"] == 2          # one 4 MiB run
+        kvm.set_option("swap_kernel_below", 0)
+        assert kvm.swap_plan(*scattered, 1024)["mode"] == 2
+    finally:
+        kvm.set_option("swap_kernel_below", 1 << 32)
     # forced modes are reported as they are
     for mode in (0, 1, 2):
         kvm.set_option("swap_mode", mode)
         assert kvm.swap_plan(*scattered, 4 << 20)["mode"] == mode
     kvm.set_option("swap_mode", 3)
-    kvm.set_option("swap_kernel_below", 0)
-    assert kvm.swap_plan(*scattered, 1024)["mode"] == 2
-    kvm.set_option("swap_kernel_below", 2 << 20)
     with pytest.raises(kvm.KvmError) as e:
         kvm.swap_plan([0], [0], 0)
     assert e.value.code == kvm.KVM_EINVAL

@@ -191,3 +191,46 @@ def test_requests_of_a_second_context_instance_carry_its_id_to_every_worker(engi
     assert calls == [("migrate", 0, [1, 2])] * 2 + [("migrate", 4, [0, 1])] * 2
     with pytest.raises(AssertionError, match="one context instance"):
         dec2._migrate_blocks_batched([ctx.on_prefill_finished(a), mb])
+
+
+def test_a_response_of_the_reference_shape_decodes_into_the_plots_five_stages():
+    """The committed fixture is a response as the reference's API server returns it; the
+    events decode, encode back to the same records, and split into the stages of the
+    reference's latency-breakdown plot, "Transmission" being migration_end - migration_begin."""
+    import json
+    import os
+
+    from distserve_amd.lifetime import (STAGES, LifetimeEventType, json_decode_lifetime_events,
+                                        json_encode_lifetime_events, stage_seconds, transmission_seconds)
+
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "lifetime_events_response.json")
+    fixture = json.load(open(path))
+    response = fixture["response"]
+    assert sorted(response) == ["lifetime_events", "text", "timestamps"]
+    events = json_decode_lifetime_events(response["lifetime_events"])
+    assert [e.event_type for e in events] == list(LifetimeEventType)
+    assert json_encode_lifetime_events(events) == response["lifetime_events"]
+    stages = dict(zip(STAGES, stage_seconds(events)))
+    assert set(stages) == set(fixture["expected_stage_seconds"])
+    for name, want in fixture["expected_stage_seconds"].items():
+        assert stages[name] == pytest.approx(want, abs=1e-9), name
+    assert transmission_seconds(events) == pytest.approx(0.0005, abs=1e-9)
+    # the stages tile the request's life
+    assert sum(stages.values()) == pytest.approx(1001.125 - 1000.0, abs=1e-9)
+    # the events this build's hand-off stamps take the place of the fixture's two
+    ctx_model = ModelConfig.from_kv_shape(8, 8, 16)
+    dec = DecodingStageLLMEngine(ctx_model, ParallelConfig(1, 0, 1, 0), CacheConfig(16, 128), worker_factory=FakeWorker)
+    ctx = ContextStageLLMEngine(ctx_model, ParallelConfig(1, 0, 1, 0), CacheConfig(16, 128), worker_factory=FakeWorker)
+    ctx._init_kvcache(8, 0)
+    dec._init_kvcache(8, 0)
+    req = create_request(20, 5)
+    ctx.block_manager.allocate_blocks(req)
+    dec._migrate_blocks(ctx.on_prefill_finished(req))
+    mine = json_encode_lifetime_events(dec.get_and_pop_request_lifetime_events(5))
+    assert [sorted(d) for d in mine] == [sorted(d) for d in response["lifetime_events"][3:5]]
+    assert [d["event_type"] for d in mine] == [d["event_type"] for d in response["lifetime_events"][3:5]]
+    merged = response["lifetime_events"][:3] + [
+        {"timestamp": 1000.625, "event_type": mine[0]["event_type"]},
+        {"timestamp": 1000.625 + (mine[1]["timestamp"] - mine[0]["timestamp"]), "event_type": mine[1]["event_type"]},
+    ] + response["lifetime_events"][5:]
+    assert len(stage_seconds(json_decode_lifetime_events(merged))) == 5

@@ -469,3 +469,63 @@ def test_tokens_written_by_the_producer_come_back_token_for_token(kvm):
     dec._remote_call_all_workers_async("wait_for_all_swap_in")
     check("gpu")
     kvm.reset()
+
+
+class _TimedWorker(Worker):
+    """A worker that brackets its migrate call with timing events on the launch stream."""
+
+    def migrate_blocks(self, *args, **kwargs):
+        self.copy_start = torch.cuda.Event(enable_timing=True)
+        self.copy_stop = torch.cuda.Event(enable_timing=True)
+        self.copy_start.record(torch.cuda.current_stream())
+        super().migrate_blocks(*args, **kwargs)
+        self.copy_stop.record(torch.cuda.current_stream())
+
+
+@pytest.mark.parametrize("gpu_complete", [True, False], ids=["stamped-after-the-copy", "stamped-at-enqueue"])
+def test_transmission_from_lifetime_events_covers_the_copy_only_when_asked_to(kvm, gpu_complete):
+    """MigrationEnd - MigrationBegin is what the reference's plots call "Transmission"
+    (evaluation/ae-scripts/e2e/_plot.py:323-341).  With gpu_complete_lifetime_events the
+    decoding engine waits for the copy before it stamps MigrationEnd, so the interval is at
+    least the copy's own duration (HIP events around the launch) and exceeds it by host work
+    only; without, it is stamped when the asynchronous call returns and covers the enqueue."""
+    from distserve_amd.lifetime import json_encode_lifetime_events, transmission_seconds
+
+    kvm.reset()
+    model = ModelConfig.from_kv_shape(num_layers=32, num_heads=32, head_dim=128)      # 8 MiB per block, K+V
+    cache = CacheConfig(16, 256)
+    ctx = ContextStageLLMEngine(model, ParallelConfig(), cache)
+    dec = DecodingStageLLMEngine(model, ParallelConfig(), cache, worker_factory=_TimedWorker,
+                                 clear_migrated_blocks_callback=ctx.clear_migrated_blocks_callback,
+                                 gpu_complete_lifetime_events=gpu_complete)
+    ctx._init_kvcache(160, 0)
+    dec._init_kvcache(160, 0)
+    dec.register_kvcache_mem_handles(ctx.parallel_config, ctx.kv_cache_mem_handles)
+    fill(ctx.workers[0][0], 77)
+    dw = dec.workers[0][0]
+    transmissions, copies = [], []
+    for rid in range(4):                                   # the first request warms everything up
+        req = create_request(2048, rid)                    # 128 blocks = 1 GiB, about 0.3 ms of copy
+        ctx.block_manager.allocate_blocks(req)
+        req.add_generated_token("x", 1)
+        m = ctx.on_prefill_finished(req)
+        ci = list(m.block_indexes)
+        torch.cuda.synchronize()
+        dec._migrate_blocks(m)
+        di = dec.block_manager.get_block_table(rid)
+        torch.cuda.synchronize()
+        events = dec.get_and_pop_request_lifetime_events(rid)
+        assert [d["event_type"] for d in json_encode_lifetime_events(events)] == ["migration_begin", "migration_end"]
+        transmissions.append(transmission_seconds(events))
+        copies.append(dw.copy_start.elapsed_time(dw.copy_stop) * 1e-3)
+        assert torch.equal(dw.k_cache[di].view(torch.int16), ctx.workers[0][0].k_cache[ci].view(torch.int16))
+        dec.block_manager.free_blocks(rid)
+    for t, c in zip(transmissions[1:], copies[1:]):
+        assert 150e-6 < c < 2e-3, c                        # 2 GiB of traffic at 1-14 TB/s: the copy was really timed
+        if gpu_complete:
+            # two clocks (host wall clock, GPU events): allow a few microseconds between them
+            assert t >= c - 20e-6, (t, c)
+            assert t <= c + 1.5e-3, (t, c)                 # the rest is host work: call, wait, wake-up
+        else:
+            assert t < c, (t, c)                           # stamped while the copy was still running
+    kvm.reset()

@@ -37,7 +37,7 @@ def run_bench(*flags, timeout=300):
 
 
 def test_migration_line_meets_the_contract_and_the_target():
-    line = run_bench("--steps", "10", "--warmup", "3")
+    line = run_bench("--steps", "10", "--warmup", "3", timeout=600)
     for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better",
                 "scaling", "vs_baseline", "dtype", "data", "config", "roofline", "cpu_baseline"):
         assert key in line, key
@@ -53,6 +53,24 @@ def test_migration_line_meets_the_contract_and_the_target():
     cpu = line["cpu_baseline"]
     assert cpu["kind"] == "port" and cpu["unit"] == "GB/s" and cpu["cores"] >= 1 and cpu["value"] > 0 and cpu["sample"]
     assert roof["frac"] >= 0.75, f"migration at {roof['frac']:.3f} of the HBM peak"
+    assert "traffic_source" in roof and "profiles/" in roof["traffic_source"]
+    assert 0 < line["host_call_us"] < 100                     # one call on an idle stream: microseconds
+    # every other configuration rides along in the same line
+    configs = line["configs"]
+    assert sorted(configs) == ["cfg1", "cfg2_batched", "cfg3", "cfg3_batched", "cfg4", "cfg4_batched", "cfg5"]
+    for name in ("cfg1", "cfg2_batched", "cfg3", "cfg3_batched", "cfg4", "cfg4_batched"):
+        c = configs[name]
+        assert c["bit_exact"] is True, name
+        for key in ("GBps", "frac", "us_per_request", "blocks_per_s", "pattern", "kernel"):
+            assert key in c, (name, key)
+        assert abs(c["frac"] - c["GBps"] / 8000.0) < 1e-3
+    assert configs["cfg1"].get("cache_resident") is True and "cache_resident" not in configs["cfg3"]
+    assert configs["cfg3"]["frac"] >= 0.75 and configs["cfg4"]["frac"] >= 0.70
+    swap = configs["cfg5"]
+    assert swap["bit_exact"] is True
+    for phase in ("alone", "beside_8_requests", "beside_continuous_migration"):
+        assert swap[phase]["swap_out_frac_of_link"] >= 0.80 and swap[phase]["swap_in_frac_of_link"] >= 0.80, (phase, swap)
+    assert swap["host_enqueue_us"]["swap_out_beside_8_requests"] <= 1000
 
 
 def test_swap_line_meets_the_target():
