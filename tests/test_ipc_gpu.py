@@ -26,12 +26,15 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CHILD = os.path.join(HERE, "ipc_context_child.py")
 
 
-class ContextProcess:
-    """The child and a line-at-a-time conversation with it; every wait has a limit."""
+DECODING_CHILD = os.path.join(HERE, "ipc_decoding_child.py")
 
-    def __init__(self, spec: dict, log_path: str):
+
+class ContextProcess:
+    """A child and a line-at-a-time conversation with it; every wait has a limit."""
+
+    def __init__(self, spec: dict, log_path: str, script: str = CHILD):
         self.log = open(log_path, "w")
-        self.proc = subprocess.Popen([sys.executable, "-u", CHILD], stdin=subprocess.PIPE, stdout=subprocess.PIPE,
+        self.proc = subprocess.Popen([sys.executable, "-u", script], stdin=subprocess.PIPE, stdout=subprocess.PIPE,
                                      stderr=self.log, text=True, cwd=os.path.dirname(HERE))
         self.lines: "queue.Queue[str]" = queue.Queue()
         threading.Thread(target=self._pump, daemon=True).start()
@@ -52,7 +55,17 @@ class ContextProcess:
             line = ""
         if not line:
             self.close(kill=True)
-            raise AssertionError("the context process did not answer; its stderr:\n" + open(self.log_path).read()[-3000:])
+            raise AssertionError("the child process did not answer; its stderr:\n" + open(self.log_path).read()[-3000:])
+        return json.loads(line)
+
+    def read(self, timeout: float = 60) -> dict:
+        """The next line the child prints without having been asked."""
+        try:
+            line = self.lines.get(timeout=timeout)
+        except queue.Empty:
+            line = ""
+        if not line:
+            raise AssertionError("the child process said nothing more; its stderr:\n" + open(self.log_path).read()[-3000:])
         return json.loads(line)
 
     def close(self, kill: bool = False):
@@ -157,6 +170,47 @@ def test_context_instance_in_another_process_tp2pp2_to_tp4_every_rank_against_or
         ctx.close()
         kvm.reset()
     assert ctx.proc.returncode == 0, open(ctx.log_path).read()[-3000:]
+
+
+def test_context_and_decoding_instances_as_sibling_processes(kvm, tmp_path):
+    """The deployed topology: neither instance is this process.  One child holds the TP2/PP2
+    context pools, a second child binds their handles, pulls every request into its TP4
+    pools and reports a digest of each; this process only carries the JSON between them and
+    checks the digests against the oracle's pools."""
+    import hashlib
+
+    spec = dict(SPEC, seed=410, prompts=[64, 23, 120])
+    ctx = ContextProcess(spec, str(tmp_path / "context_process.log"))
+    dec = None
+    try:
+        tables = {int(k): v for k, v in ctx.hello["tables"].items()}
+        requests = [[rid, spec["prompts"][rid], tables[rid]] for rid in sorted(tables)]
+        dec = ContextProcess({"layers": 8, "kv_heads": 8, "head_dim": 64, "tp": 4, "blocks": 32, "busy_prompt": 20,
+                              "ctx_tp": 2, "ctx_pp": 2, "handles": ctx.hello["handles"], "requests": requests},
+                             str(tmp_path / "decoding_process.log"), script=DECODING_CHILD)
+        answer = dec.hello
+        assert len({os.getpid(), ctx.hello["pid"], answer["pid"]}) == 3
+        assert 1 <= answer["opened"] <= 8
+        src_k, src_v = child_sources(spec)
+        shape = oracle.Geom(8, 8, 16, 64, 2, 2, 2, 1, 4).dec_pool_shape(32)
+        for u in range(4):
+            g = oracle.Geom(8, 8, 16, 64, 2, 2, 2, 1, 4, 0, u)
+            for src, got in ((src_k, answer["digests"][u][0]), (src_v, answer["digests"][u][1])):
+                want = canary_pool(shape)
+                for rid, _, ctx_table in requests:
+                    oracle.migrate_c(g, src, ctx_table, answer["tables"][str(rid)], want)
+                assert hashlib.sha256(oracle.bits(want).numpy().tobytes()).hexdigest() == got, u
+        assert ctx.ask({"cmd": "verify"}, timeout=120)["unchanged"] is True
+        dec.proc.stdin.write(json.dumps({"cmd": "exit"}) + "\n")
+        dec.proc.stdin.flush()
+        assert dec.read()["opened_after_reset"] == 0
+        dec.proc.wait(timeout=60)
+    finally:
+        if dec is not None:
+            dec.close()
+        ctx.close()
+    assert ctx.proc.returncode == 0 and dec.proc.returncode == 0, (
+        open(ctx.log_path).read()[-2000:] + open(dec.log_path).read()[-2000:])
 
 
 def test_own_handles_still_resolve_without_ipc_whatever_the_pool_size(kvm):
