@@ -148,6 +148,24 @@ class ModelConfig:
             f"tensor parallel group ({tp}).")
         return total // tp
 
+    def kv_heads_replicated(self, parallel_config: ParallelConfig = ParallelConfig()) -> bool:
+        """True when every tensor rank holds a copy of the same KV head instead of a slice of
+        them: a multi-query model under tensor parallelism (reference config.py:233-237
+        returns 1 head per rank whatever the tensor-parallel size)."""
+        tp = parallel_config.tensor_parallel_size
+        return tp > 1 and self.get_num_heads(parallel_config) * tp != self.get_num_heads()
+
+    def check_kv_heads_are_split(self, parallel_config: ParallelConfig) -> None:
+        """The migration re-slices KV heads between tensor ranks that each own a contiguous
+        slice ``[t*H/T, (t+1)*H/T)``.  Replicated heads have no such slice: which copy a
+        decoding rank should read is a choice the reference's native op makes and its sources
+        do not show, so that layout is refused here instead of guessed."""
+        if self.kv_heads_replicated(parallel_config):
+            raise ValueError(
+                f"model {self.model!r} keeps {self.get_num_heads()} KV head(s) replicated on each of "
+                f"{parallel_config.tensor_parallel_size} tensor ranks (multi-query attention); KV migration "
+                "between instances needs KV heads that are split over the tensor ranks")
+
     def get_num_layers(self, parallel_config: ParallelConfig = ParallelConfig()) -> int:
         """Layers held by one pipeline rank (reference config.py:279-286)."""
         total = self.hf_config.num_hidden_layers

@@ -40,6 +40,7 @@ class Worker:
                  parallel_config: ParallelConfig = ParallelConfig(),
                  tensor_parallel_id: List[int] = None, pipeline_parallel_id: List[int] = None,
                  forward: Optional[Callable] = None) -> None:
+        model_config.check_kv_heads_are_split(parallel_config)
         _require_gpu()
         self.worker_id = worker_id
         self.stage = stage
