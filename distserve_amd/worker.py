@@ -12,8 +12,8 @@ Ordering differs from the reference where the reference is unsafe, never in what
   before, worker.py:286-287 vs :302-311, so its event does not cover the copy);
 * a side stream first waits for the work already enqueued on the compute stream, so a
   swap-out never reads a block the forward pass is still writing;
-* ``migrate_blocks`` leaves an event (``latest_migrate_event``) that the context instance
-  waits on before it reuses the freed source blocks.
+* ``migrate_blocks`` leaves a mark (``latest_migrate_event``) that the context instance
+  makes its stream wait on before it reuses the freed source blocks.
 """
 from __future__ import annotations
 
@@ -31,6 +31,35 @@ from distserve_amd.utils import MemoryHandle, Stage
 def _require_gpu() -> None:
     if not torch.cuda.is_available():
         raise RuntimeError("distserve_amd.Worker needs a GPU: the KV movement path has no CPU fallback")
+
+
+class MigrationMark:
+    """Stands for "the copies enqueued on ``stream`` so far" with the interface of an event
+    (``wait``, ``synchronize``, ``query``).  The HIP event behind it is only recorded when
+    somebody needs one: work that follows on the same stream is behind the copies by stream
+    order alone, and that is the common case (one worker thread, one current stream), where
+    an eager event per migrated request would be two runtime calls that order nothing.  An
+    event recorded late covers the copies all the same (and whatever the stream got since)."""
+
+    def __init__(self, stream: torch.cuda.Stream):
+        self.stream = stream
+        self._event: Optional[torch.cuda.Event] = None
+
+    def _recorded(self) -> torch.cuda.Event:
+        if self._event is None:
+            self._event = torch.cuda.Event()
+            self._event.record(self.stream)
+        return self._event
+
+    def wait(self, stream: torch.cuda.Stream) -> None:
+        if stream != self.stream:
+            self._recorded().wait(stream)
+
+    def synchronize(self) -> None:
+        self._recorded().synchronize()
+
+    def query(self) -> bool:
+        return self._recorded().query()
 
 
 class Worker:
@@ -63,7 +92,7 @@ class Worker:
         self.swap_event_table: Dict[int, torch.cuda.Event] = {}   # request_id -> its latest swap
         self.latest_swap_in_event: Optional[torch.cuda.Event] = None
         self.latest_swap_out_event: Optional[torch.cuda.Event] = None
-        self.latest_migrate_event: Optional[torch.cuda.Event] = None
+        self.latest_migrate_event: Optional[MigrationMark] = None
         self.execution_time = 0.0
         self.blocked_swapping_time = 0.0
 
@@ -173,11 +202,9 @@ class Worker:
             self.k_cache,
             self.v_cache,
         )
-        event = torch.cuda.Event()
-        event.record(self._current_stream())
-        self.latest_migrate_event = event
+        self.latest_migrate_event = MigrationMark(self._current_stream())
 
-    def wait_stream_for_migration(self, event: Optional[torch.cuda.Event]) -> None:
+    def wait_stream_for_migration(self, event: Optional[MigrationMark]) -> None:
         """Called on a *context* worker: work it enqueues from now on (the next prefill that
         may overwrite freed blocks) runs after the migration that read them."""
         if event is not None:

@@ -39,3 +39,31 @@ def make_src_pools(g: oracle.Geom, num_blocks: int, seed: int, dtype=torch.float
 
 def same_bits(a: torch.Tensor, b: torch.Tensor) -> bool:
     return a.shape == b.shape and torch.equal(oracle.bits(a.contiguous()), oracle.bits(b.contiguous()))
+
+
+def labelled_src_pools(g: oracle.Geom, num_blocks: int, dtype=torch.int32) -> List[List[torch.Tensor]]:
+    """Context pools whose every element carries its own global coordinates:
+    ``label = ((block * L + layer) * H + head) * (B*D) + slot`` with the layer and head counted
+    over the WHOLE model.  Built from the rank -> slice rule alone (rank p of P holds layers
+    [p*L/P, (p+1)*L/P), rank t of T heads [t*H/T, (t+1)*H/T)), with no copy arithmetic."""
+    L, H, BD = g.num_layers, g.num_kv_heads, g.block_size * g.head_dim
+    whole = torch.arange(num_blocks * L * H * BD, dtype=torch.int64).view(num_blocks, L, H, g.block_size, g.head_dim)
+    Lc, Hc = L // g.ctx_pp, H // g.ctx_tp
+    return [[whole[:, p * Lc:(p + 1) * Lc, t * Hc:(t + 1) * Hc].contiguous().to(dtype)
+             for t in range(g.ctx_tp)] for p in range(g.ctx_pp)]
+
+
+def expected_labels(g: oracle.Geom, ci, di, nb_dst: int, fill: int, dtype=torch.int32) -> torch.Tensor:
+    """What the decoding rank's pool must hold after migrating labelled pools: at decoding
+    block di[i], local (layer, head), the label of context block ci[i] and the GLOBAL layer
+    and head that this rank's local ones stand for; ``fill`` everywhere else."""
+    L, H, BD = g.num_layers, g.num_kv_heads, g.block_size * g.head_dim
+    Ld, Hd = L // g.dec_pp, H // g.dec_tp
+    out = torch.full((nb_dst, Ld, Hd, g.block_size, g.head_dim), fill, dtype=torch.int64)
+    slot = torch.arange(BD).view(g.block_size, g.head_dim)
+    for c, d in zip(ci, di):
+        for l in range(Ld):
+            for h in range(Hd):
+                gl, gh = g.dec_pp_rank * Ld + l, g.dec_tp_rank * Hd + h
+                out[d, l, h] = ((c * L + gl) * H + gh) * BD + slot
+    return out.to(dtype)

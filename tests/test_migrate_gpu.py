@@ -64,6 +64,30 @@ def test_layouts_whose_splits_do_not_nest(kvm, cpp, ctp, dpp, dtp):
             check_case(kvm, g, 5, 6, ci, di, seed=17)
 
 
+@pytest.mark.parametrize("cpp,ctp,dpp,dtp", [(2, 2, 1, 4), (1, 2, 1, 1), (4, 1, 2, 2), (2, 4, 4, 1), (3, 2, 2, 3), (1, 6, 3, 4)])
+def test_labelled_elements_arrive_under_their_global_layer_and_head(kvm, cpp, ctp, dpp, dtp):
+    """The kernel against expectations written down without any copy arithmetic: every source
+    element carries its global (block, layer, head, slot), and the destination must hold, at
+    decoding block di[i], the labels of context block ci[i] for this rank's layers and heads."""
+    from helpers import expected_labels, labelled_src_pools
+
+    ci, di = [4, 0, 2, 3], [1, 6, 3, 0]
+    for q in range(dpp):
+        for u in range(dtp):
+            g = oracle.Geom(12, 12, 16, 8, 4, cpp, ctp, dpp, dtp, q, u)
+            kvm.reset()
+            src = labelled_src_pools(g, 5)
+            keep = upload_and_register(g, src, src)
+            dst_k = torch.full(g.dec_pool_shape(7), -7, dtype=torch.int32, device="cuda")
+            dst_v = torch.full(g.dec_pool_shape(7), -7, dtype=torch.int32, device="cuda")
+            kvm.migrate(kvm_geom(g), ci, di, dst_k.data_ptr(), dst_v.data_ptr(), 7, stream_handle())
+            torch.cuda.synchronize()
+            want = expected_labels(g, ci, di, 7, fill=-7)
+            assert torch.equal(dst_k.cpu(), want) and torch.equal(dst_v.cpu(), want), (q, u)
+            del keep
+    kvm.reset()
+
+
 def test_golden_fixtures(kvm):
     import hashlib
     from golden.make_golden import build_case

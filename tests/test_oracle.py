@@ -64,6 +64,28 @@ def test_three_formulations_agree_when_the_splits_do_not_nest(cpp, ctp, dpp, dtp
             assert same_bits(a, b) and same_bits(a, c)
 
 
+@pytest.mark.parametrize("cpp,ctp,dpp,dtp", list(_layouts()) + _uneven_layouts(12, seed=9))
+def test_labelled_elements_arrive_under_their_global_layer_and_head(cpp, ctp, dpp, dtp):
+    """Every element of the context pools carries its global (block, layer, head, slot) as
+    its value, so the expected destination is written down from the meaning of the copy
+    alone -- "decoding block di[i] holds context block ci[i]'s layers and heads of this
+    rank" -- with none of the oracle's offset arithmetic.  A wrong owner, a wrong local
+    offset, a transposed layer/head or a dropped rank all show as a wrong label."""
+    from helpers import expected_labels, labelled_src_pools
+
+    L = H = 12 if 3 in (cpp, ctp, dpp, dtp) or 6 in (cpp, ctp, dpp, dtp) else 4
+    ci, di = [4, 0, 2], [1, 6, 3]
+    for q in range(dpp):
+        for u in range(dtp):
+            g = oracle.Geom(L, H, 2, 3, 4, cpp, ctp, dpp, dtp, q, u)
+            src = labelled_src_pools(g, 5)
+            want = expected_labels(g, ci, di, 7, fill=-7)
+            for fn in (oracle.migrate_c, oracle.migrate_cat):
+                dst = torch.full(g.dec_pool_shape(7), -7, dtype=torch.int32)
+                fn(g, src, ci, di, dst)
+                assert torch.equal(dst, want), (fn.__name__, q, u)
+
+
 def test_tp1_pp1_reduces_to_index_copy_of_index_select():
     g = oracle.Geom(3, 5, 4, 8, 2)
     src = make_src_pools(g, 9, seed=3)

@@ -529,3 +529,52 @@ def test_transmission_from_lifetime_events_covers_the_copy_only_when_asked_to(kv
         else:
             assert t < c, (t, c)                           # stamped while the copy was still running
     kvm.reset()
+
+
+def test_freed_source_blocks_are_reused_only_after_a_migration_on_another_stream_has_read_them(kvm):
+    """The decoding worker pulls on a side stream; the context worker, on the default stream,
+    makes its stream wait on the migration's mark and then overwrites the freed blocks (the
+    next prefill would).  The destination must hold what the blocks held before.  On one and
+    the same stream the mark costs nothing: no event is recorded."""
+    kvm.reset()
+    model = ModelConfig.from_kv_shape(num_layers=32, num_heads=32, head_dim=128)
+    cache = CacheConfig(16, 256)
+    ctx_w = Worker(0, Stage.CONTEXT, model, cache)
+    dec_w = Worker(1, Stage.DECODING, model, cache)
+    hk, hv = ctx_w.init_kvcache_and_swap(96, 1)
+    dec_w.init_kvcache_and_swap(96, 1)
+    dec_w.register_kvcache_mem_handles(ParallelConfig(), [[(hk, hv)]])
+    ctx_w.k_cache.view(torch.int16).fill_(0x1234)
+    ctx_w.v_cache.view(torch.int16).fill_(0x2345)
+    dec_w.k_cache.view(torch.int16).fill_(0x7C01)
+    dec_w.v_cache.view(torch.int16).fill_(0x7C01)
+    ci, di = list(range(10, 90)), list(range(5, 85))           # 80 blocks = 640 MiB, about 0.2 ms of copy
+    side = torch.cuda.Stream()
+    torch.cuda.synchronize()
+    for attempt in range(3):
+        with torch.cuda.stream(side):
+            dec_w.migrate_blocks(ci, ParallelConfig(), di)
+        mark = dec_w.latest_migrate_event
+        assert mark._event is None                              # nothing recorded until somebody needs it
+        ctx_w.wait_stream_for_migration(mark)                   # default stream now waits for the side stream's copy
+        assert mark._event is not None
+        ctx_w.k_cache[ci] = 0                                    # the "next prefill" overwrites the freed blocks
+        ctx_w.v_cache[ci] = 0
+        torch.cuda.synchronize()
+        assert bool((dec_w.k_cache[di].view(torch.int16) == 0x1234).all()), attempt
+        assert bool((dec_w.v_cache[di].view(torch.int16) == 0x2345).all()), attempt
+        ctx_w.k_cache.view(torch.int16).fill_(0x1234)
+        ctx_w.v_cache.view(torch.int16).fill_(0x2345)
+        dec_w.k_cache.view(torch.int16).fill_(0x7C01)
+        torch.cuda.synchronize()
+    # same stream: ordering is the stream's own, and the mark stays unrecorded
+    dec_w.migrate_blocks(ci, ParallelConfig(), di)
+    mark = dec_w.latest_migrate_event
+    ctx_w.wait_stream_for_migration(mark)
+    assert mark._event is None
+    ctx_w.k_cache[ci] = 0
+    torch.cuda.synchronize()
+    assert bool((dec_w.k_cache[di].view(torch.int16) == 0x1234).all())
+    mark.synchronize()                                          # asked for, it is a real event
+    assert mark._event is not None and mark.query() is True
+    kvm.reset()
