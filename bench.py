@@ -232,6 +232,11 @@ def bench_migrate(config: int, pattern: str, steps: int, warmup: int, verify_res
 
     for _ in range(warmup):
         step()
+    # no collector pass inside the timed region (a full one over torch's modules takes 35 ms)
+    import gc
+
+    gc.collect()
+    gc.freeze()
     torch.cuda.synchronize()
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     start.record(stream)
