@@ -772,10 +772,9 @@ int launch_copy(std::vector<Seg> segs, const IdxPair *pairs, int64_t n, char *ds
         if (walk_wgs > 0) {
             max_items = std::max<int64_t>(max_items, 2 * 256 * (int64_t)walk_wgs);
         } else {
-            MigrateArgs probe = args;
-            probe.nidx = (uint32_t)largest;
-            plan_work(probe, grp.tiles, tile_bytes);
-            const int64_t items = 2 * (int64_t)probe.work_padded * k.threads;
+            args.nidx = (uint32_t)largest;      // the launch loop below sets it again, launch by launch
+            plan_work(args, grp.tiles, tile_bytes);
+            const int64_t items = 2 * (int64_t)args.work_padded * k.threads;
             if (items > (int64_t)UINT32_MAX)
                 return fail(KVM_EINVAL, "a launch of %lld work-items cannot be made", (long long)items);
             max_items = std::max(max_items, items);
@@ -1074,6 +1073,14 @@ static int open_handle(const int64_t *h, const char *what, const char **ptr, int
         (void)hipGetLastError();
         return fail(KVM_EHANDLE, "%s handle of process %lld could not be opened: %s", what, (long long)h[kHwPid],
                     hipGetErrorString(e));
+    }
+    // The size in the handle is the exporter's word; where the runtime can tell how much it
+    // has mapped, a handle that claims more is refused before a kernel could run off the end.
+    const uint64_t mapped = extent_of(local);
+    if (mapped != 0 && mapped < (uint64_t)h[kHwAllocSize]) {
+        (void)hipIpcCloseMemHandle(local);
+        return fail(KVM_EHANDLE, "%s handle of process %lld says its allocation holds %lld bytes, the mapping holds %llu",
+                    what, (long long)h[kHwPid], (long long)h[kHwAllocSize], (unsigned long long)mapped);
     }
     g_opened.push_back(Opened{h[kHwPid], h[kHwAllocBase], h[kHwAllocSize], ipc, (char *)local});
     *ptr = (char *)local + off;
