@@ -2,6 +2,7 @@
 
 ``libkvmove.so``        hand-written HIP kernels + the C ABI (``include/kvmove.h``); no torch.
 ``libkvmove_torch.so``  torch op shim registering ``block_migration_ops`` / ``swapping_ops``.
+``hbm_probe``           stand-alone program: what plain one-shot kernels reach on the copy's address patterns.
 ``libkvmove_torch_alt.so``  the same ops as ``kvmove_block_migration_ops`` / ``kvmove_swapping_ops``,
                         for a process that keeps another registration of DistServe's names.
 
@@ -25,6 +26,7 @@ INCLUDE_DIR = os.path.join(REPO_DIR, "include")
 KVMOVE_LIB = os.path.join(LIB_DIR, "libkvmove.so")
 TORCH_LIB = os.path.join(LIB_DIR, "libkvmove_torch.so")
 TORCH_ALT_LIB = os.path.join(LIB_DIR, "libkvmove_torch_alt.so")
+HBM_PROBE = os.path.join(LIB_DIR, "hbm_probe")
 ALT_NAMESPACES = ("kvmove_block_migration_ops", "kvmove_swapping_ops")
 
 GPU_ARCH = "gfx950"
@@ -54,6 +56,18 @@ def build_kvmove() -> str:
     return KVMOVE_LIB
 
 
+def build_hbm_probe() -> str:
+    """The stand-alone ceiling probe (``hbm_probe.hip``): a program, not part of the library."""
+    hipcc = shutil.which("hipcc") or os.path.join(ROCM_HOME, "bin", "hipcc")
+    os.makedirs(LIB_DIR, exist_ok=True)
+    _run([
+        hipcc, f"--offload-arch={GPU_ARCH}", "-O3", "-std=c++17",
+        "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wall", "-Wextra",
+        os.path.join(CSRC_DIR, "hbm_probe.hip"), "-o", HBM_PROBE,
+    ])
+    return HBM_PROBE
+
+
 def build_torch_shim(alt: bool = False) -> str:
     import torch
     from torch.utils import cpp_extension
@@ -81,9 +95,10 @@ def build_all() -> None:
     build_kvmove()
     build_torch_shim()
     build_torch_shim(alt=True)
+    build_hbm_probe()
 
 
 if __name__ == "__main__":
     build_all()
-    print("built:", KVMOVE_LIB, TORCH_LIB, TORCH_ALT_LIB)
+    print("built:", KVMOVE_LIB, TORCH_LIB, TORCH_ALT_LIB, HBM_PROBE)
     sys.exit(0)

@@ -206,3 +206,17 @@ def test_the_alternate_namespace_build_registers_the_same_schemas_beside_the_fir
         assert args_of(getattr(torch.ops.kvmove_block_migration_ops, name)) == \
             args_of(getattr(torch.ops.block_migration_ops, name))
     assert args_of(torch.ops.kvmove_swapping_ops.swap) == args_of(torch.ops.swapping_ops.swap)
+
+
+def test_the_ceiling_probe_is_built_and_explains_its_flags():
+    """The stand-alone probe of the memory system's ceilings is built beside the libraries
+    (no GPU call happens before its arguments are read)."""
+    import subprocess
+
+    import distserve_amd
+
+    probe = os.path.join(os.path.dirname(distserve_amd.TORCH_LIB_PATH), "hbm_probe")
+    assert os.path.exists(probe), "python distserve_amd/csrc/build.py builds it"
+    run = subprocess.run([probe, "--no-such-flag"], capture_output=True, text=True)
+    assert run.returncode == 2
+    assert "--section" in run.stderr and "--quick" in run.stderr
