@@ -110,9 +110,11 @@ __global__ __launch_bounds__(THREADS) void probe_kernel(const ProbeArgs a)
 // The copy with block tables, at a fixed geometry and nothing else: block b of the launch is
 // NSEG segments of ROWS rows of ROW_TILES one-KiB tiles; segment j of it is read from block
 // src_ids[b] of source pool j, where a row starts every ROW_STRIDE_TILES KiB, and the block
-// is written densely to block dst_ids[b] of the destination pool.  <8, 16, 40, 2> is one pool
-// kind of a request of the 70B configuration (two of four heads from each of two pipeline
-// stages); <8, 8, 40, 2> is the same bytes from pools that hold exactly those two heads.
+// is written densely to block dst_ids[b] of the destination pool.  <8, 16, 40, 2, false> is
+// one pool kind of a request of the 70B configuration (two of four heads from each of two
+// pipeline stages); <8, 8, 40, 2, false> is the same bytes from pools that hold exactly
+// those two heads; <80, 80, 40, 2, true> is the 13B configuration (each of 40 layer rows is
+// 80 KiB from each of two tensor-parallel ranks, side by side).
 struct TableArgs {
     char *dst;
     const char *src[2];
@@ -122,7 +124,7 @@ struct TableArgs {
     uint32_t pad;
 };
 
-template <int ROW_TILES, int ROW_STRIDE_TILES, int ROWS, int NSEG>
+template <int ROW_TILES, int ROW_STRIDE_TILES, int ROWS, int NSEG, bool INTERLEAVED>
 __global__ __launch_bounds__(64) void table_kernel(const TableArgs a)
 {
     constexpr uint32_t kBlockTiles = ROW_TILES * ROWS * NSEG, kSegTiles = ROW_TILES * ROWS;
@@ -133,9 +135,20 @@ __global__ __launch_bounds__(64) void table_kernel(const TableArgs a)
         t = (q * 8u + xcd) * a.chunk_tiles + (seq - q * a.chunk_tiles);
     }
     if (t >= a.tiles) return;
+    // u: the tile's place in the destination block, which is written densely
     const uint32_t b = t / kBlockTiles, u = t - b * kBlockTiles;
-    const uint32_t seg = u / kSegTiles, v = u - seg * kSegTiles;
-    const uint32_t row = v / ROW_TILES, within = v - row * ROW_TILES;
+    uint32_t seg, row, within;
+    if constexpr (INTERLEAVED) {   // a destination row is the segments' rows side by side
+        row = u / (ROW_TILES * NSEG);
+        const uint32_t v = u - row * (ROW_TILES * NSEG);
+        seg = v / ROW_TILES;
+        within = v - seg * ROW_TILES;
+    } else {                       // the segments follow each other
+        seg = u / kSegTiles;
+        const uint32_t v = u - seg * kSegTiles;
+        row = v / ROW_TILES;
+        within = v - row * ROW_TILES;
+    }
     const uint64_t sblock = (uint64_t)(uint32_t)a.src_ids[b] * (ROW_STRIDE_TILES * ROWS * 1024u);
     const uint64_t dblock = (uint64_t)(uint32_t)a.dst_ids[b] * (kBlockTiles * 1024u);
     const uint64_t saddr = (uint64_t)a.src[seg] + sblock + row * (ROW_STRIDE_TILES * 1024u) + a.src_row_off +
@@ -234,11 +247,10 @@ static Result run_case(const Flavour &f, Mode mode, char *dst, const char *src, 
 
 // Block-table copies: `launches` launches of `nb` blocks each, lists sequential (advancing
 // through the pools) or random (no block twice in a launch), back to back.
-template <int ROW_TILES, int ROW_STRIDE_TILES, int ROWS, int NSEG>
-static Result run_table(char *dst, const char *src, uint32_t nb, bool src_random, bool dst_random, int chunk_mode,
-                        int launches)
+template <int ROW_TILES, int ROW_STRIDE_TILES, int ROWS, int NSEG, bool INTERLEAVED>
+static Result run_table(char *dst, const char *src, uint32_t src_blocks, uint32_t dst_blocks, uint32_t nb,
+                        bool src_random, bool dst_random, int chunk_mode, int launches)
 {
-    constexpr uint32_t kSrcBlocks = 1024, kDstBlocks = 2048;
     constexpr uint32_t kBlockTiles = ROW_TILES * ROWS * NSEG;
     const int passes = 3, total_launches = (passes + 1) * launches;
     std::vector<int32_t> sid((size_t)total_launches * nb), did((size_t)total_launches * nb);
@@ -258,8 +270,8 @@ static Result run_table(char *dst, const char *src, uint32_t nb, bool src_random
             off += nb;
         }
     };
-    fill(sid, kSrcBlocks, src_random);
-    fill(did, kDstBlocks, dst_random);
+    fill(sid, src_blocks, src_random);
+    fill(did, dst_blocks, dst_random);
     int32_t *d_sid = nullptr, *d_did = nullptr;
     CHECK(hipMalloc((void **)&d_sid, sid.size() * 4));
     CHECK(hipMalloc((void **)&d_did, did.size() * 4));
@@ -270,6 +282,12 @@ static Result run_table(char *dst, const char *src, uint32_t nb, bool src_random
     a.dst = dst;
     a.src[0] = src;
     a.src[1] = src + (4ull << 30);
+    if ((uint64_t)src_blocks * ROW_STRIDE_TILES * ROWS * 1024u > (4ull << 30) ||
+        (uint64_t)dst_blocks * kBlockTiles * 1024u > (8ull << 30) || nb > src_blocks || nb > dst_blocks ||
+        (uint64_t)nb * kBlockTiles * 64u >= (1ull << 32)) {
+        fprintf(stderr, "table case does not fit the buffers or the grid\n");
+        exit(2);
+    }
     a.tiles = nb * kBlockTiles;
     a.chunk_tiles = chunk_mode == 0 ? 0 : chunk_mode == 1 ? (a.tiles + 7) / 8 : 256;
     a.src_row_off = (ROW_STRIDE_TILES - ROW_TILES) * 1024u;   // the wanted heads are the last of the row
@@ -284,7 +302,7 @@ static Result run_table(char *dst, const char *src, uint32_t nb, bool src_random
         for (int l = 0; l < launches; ++l) {
             a.src_ids = d_sid + (size_t)(pass * launches + l) * nb;
             a.dst_ids = d_did + (size_t)(pass * launches + l) * nb;
-            hipLaunchKernelGGL((table_kernel<ROW_TILES, ROW_STRIDE_TILES, ROWS, NSEG>), dim3(grid), dim3(64), 0, nullptr, a);
+            hipLaunchKernelGGL((table_kernel<ROW_TILES, ROW_STRIDE_TILES, ROWS, NSEG, INTERLEAVED>), dim3(grid), dim3(64), 0, nullptr, a);
         }
         CHECK(hipEventRecord(e1, nullptr));
         CHECK(hipEventSynchronize(e1));
@@ -400,24 +418,30 @@ int main(int argc, char **argv)
             }
         }
     }
-    printf("\n3. Copies through block tables: blocks of 2 segments x 40 rows x 8 KiB, 1024-block source pools, 2048-block\n"
-           "   destination pool, 64 lanes x 1 vector\n");
+    printf("\n3. Copies through block tables (64 lanes x 1 vector; block ids from tables in device memory)\n"
+           "   70B: blocks of 2 segments x 40 rows x 8 KiB, one segment after the other; 1024-block source pools, 2048-block\n"
+           "        destination pool.  13B: blocks of 40 rows x (80 KiB from each of 2 pools); 1024-block pools.\n");
     printf("%-22s %-8s %-8s %-10s %-12s %12s %10s\n", "source rows", "source", "dest.", "blocks per", "workgroup", "us/launch",
            "GB/s");
     printf("%-22s %-8s %-8s %-10s %-12s\n", "", "blocks", "blocks", "launch", "ids");
     const char *chunk_name[] = {"in order", "launch/8", "256K/XCD"};
-    for (int dense = 0; dense < 2; ++dense) {
+    const char *geom_name[] = {"70B 8 KiB of 16 KiB", "70B 8 KiB of 8 KiB", "13B 2 x 80 KiB"};
+    for (int geom = 0; geom < 3; ++geom) {
         if (only && only != 3) break;
-        for (uint32_t nb : {272u, 1024u}) {
+        // per-request and long launches: 272 / 1024 blocks of 640 KiB, 72 / 864 blocks of 6.25 MiB
+        const uint32_t nbs[2] = {geom == 2 ? 72u : 272u, geom == 2 ? 864u : 1024u};
+        for (int size = 0; size < 2; ++size) {
             for (int sr = 0; sr < 2; ++sr) {
                 for (int dr = 0; dr < 2; ++dr) {
                     for (int cm = 0; cm < 3; ++cm) {
-                        const int launches = nb == 272 ? 24 : 6;
-                        const Result r = dense ? run_table<8, 8, 40, 2>(dst, src, nb, sr, dr, cm, launches)
-                                               : run_table<8, 16, 40, 2>(dst, src, nb, sr, dr, cm, launches);
-                        printf("%-22s %-8s %-8s %-10u %-12s %12.2f %10.1f\n", dense ? "8 KiB of 8 KiB" : "8 KiB of 16 KiB",
-                               sr ? "random" : "adjacent", dr ? "random" : "adjacent", nb, chunk_name[cm],
-                               r.us_per_launch, r.gbps);
+                        const uint32_t nb = nbs[size];
+                        const int launches = size == 0 ? 24 : geom == 2 ? 3 : 6;
+                        const Result r =
+                            geom == 0   ? run_table<8, 16, 40, 2, false>(dst, src, 1024, 2048, nb, sr, dr, cm, launches)
+                            : geom == 1 ? run_table<8, 8, 40, 2, false>(dst, src, 1024, 2048, nb, sr, dr, cm, launches)
+                                        : run_table<80, 80, 40, 2, true>(dst, src, 1024, 1024, nb, sr, dr, cm, launches);
+                        printf("%-22s %-8s %-8s %-10u %-12s %12.2f %10.1f\n", geom_name[geom], sr ? "random" : "adjacent",
+                               dr ? "random" : "adjacent", nb, chunk_name[cm], r.us_per_launch, r.gbps);
                         fflush(stdout);
                     }
                 }

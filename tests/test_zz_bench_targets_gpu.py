@@ -90,13 +90,14 @@ def test_migration_line_meets_the_contract_and_the_target():
     assert swap["host_enqueue_us"]["swap_out_beside_8_requests"] <= 1000
 
 
-def test_configuration_4_reaches_what_the_plainest_kernel_reaches_on_its_geometry():
+def test_configurations_3_and_4_reach_what_the_plainest_kernel_reaches_on_their_geometry():
     """The probe's block-table kernel has no segments, no index search and no division by a
     run-time value: what it reaches on configuration 4's geometry (8 KiB of every 16 KiB from
     two pools, blocks placed at random on both sides) is what the memory system gives that
     access pattern.  The migration kernel, with all its generality, must be within a few
     percent of it on the same box."""
-    rows = [r for r in probe_rows(3) if r[0] == "8 KiB of 16 KiB" and r[1] == "random" and r[2] == "random"]
+    table = probe_rows(3)
+    rows = [r for r in table if r[0] == "70B 8 KiB of 16 KiB" and r[1] == "random" and r[2] == "random"]
     per_request = [float(r[-1]) for r in rows if r[3] == "272"]
     long_launch = [float(r[-1]) for r in rows if r[3] == "1024"]
     assert len(per_request) == 3 and len(long_launch) == 3, rows
@@ -104,6 +105,11 @@ def test_configuration_4_reaches_what_the_plainest_kernel_reaches_on_its_geometr
     configs = default_line()["configs"]
     assert configs["cfg4"]["GBps"] >= 0.93 * max(per_request), (configs["cfg4"]["GBps"], per_request)
     assert configs["cfg4_batched"]["GBps"] >= 0.93 * max(long_launch), (configs["cfg4_batched"]["GBps"], long_launch)
+    # configuration 3's geometry: whole blocks, 80 KiB pieces of two pools side by side
+    rows = [r for r in table if r[0] == "13B 2 x 80 KiB" and r[1] == "random" and r[2] == "random"]
+    per_request = [float(r[-1]) for r in rows if r[3] == "72"]
+    assert len(per_request) == 3, rows
+    assert configs["cfg3"]["GBps"] >= 0.93 * max(per_request), (configs["cfg3"]["GBps"], per_request)
 
 
 def test_swap_line_meets_the_target():
