@@ -86,6 +86,15 @@ SPEC = {"layers": 8, "kv_heads": 8, "head_dim": 64, "tp": 2, "pp": 2, "blocks": 
         "busy_blocks": 3, "prompts": [40, 16, 97, 33]}
 
 
+def sealed(words) -> int:
+    """The check word of a handle, as the library computes it over the 16 words before it."""
+    mask = (1 << 64) - 1
+    x = 0x5A5A5A5A5A5A5A5A
+    for w in words[:16]:
+        x = (((x << 7) | (x >> 57)) & mask) ^ (w & mask)
+    return x - (1 << 64) if x >> 63 else x
+
+
 def child_sources(spec):
     """The pools the child holds, remade here on the CPU from the seed: src[pp][tp]."""
     import ipc_context_child as child
@@ -165,6 +174,17 @@ def test_context_instance_in_another_process_tp2pp2_to_tp4_every_rank_against_or
         with pytest.raises(kvm.KvmError) as e:
             kvm.register_mem_handle(big, big, 8, 8, [1, 0, 1, 0], [1, 0, 1, 0])
         assert e.value.code == kvm.KVM_EHANDLE and "not shared between processes" in str(e.value)
+        assert kvm.opened_handles() == 0
+
+        # a well-formed handle that claims a larger allocation than the other process holds is
+        # refused once the mapping is there to be measured, and the mapping is closed again
+        lie = list(handles[0][0][0])
+        lie[6] *= 64                                    # the allocation's size, as the exporter tells it
+        lie[4] = lie[6] - (lie[3] - lie[5])             # a pool that runs to the claimed end
+        lie[16] = sealed(lie)
+        with pytest.raises(kvm.KvmError) as e:
+            kvm.register_mem_handle(lie, lie, 8, 8, [1, 0, 1, 0], [1, 0, 1, 0])
+        assert e.value.code == kvm.KVM_EHANDLE and "the mapping holds" in str(e.value)
         assert kvm.opened_handles() == 0
     finally:
         ctx.close()
