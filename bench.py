@@ -41,9 +41,12 @@ def parse_args():
     ap.add_argument("--ctx-tp", type=int, default=0,
                     help="configuration 4 only: context tensor-parallel size. 2 is the configuration itself (8 KiB runs "
                          "at a 16 KiB source stride); 4 moves the same bytes from dense source pools, for comparison")
-    ap.add_argument("--pattern", default="request", choices=["request", "batch", "handoff", "handoff-batched"],
+    ap.add_argument("--pattern", default="request",
+                    choices=["request", "batch", "handoff", "handoff-batched", "scheduler", "scheduler-batched"],
                     help="handoff*: the same requests through Worker / BlockManager / the migration handoff "
-                         "(torch ops, block allocation and release included), one call per request or one per batch")
+                         "(torch ops, block allocation and release included), one call per request or one per batch; "
+                         "scheduler*: the same, with the decoding scheduler's post_process deciding acceptance "
+                         "(bridge queue -> scheduler -> engine -> op), batch_migrations off or on")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-verify", action="store_true")
     ap.add_argument("--opt", action="append", default=[], help="kvmove tuning option name=value")
@@ -360,7 +363,7 @@ def main():
         print(json.dumps(run_swap_bench(args)))
         return
 
-    if args.pattern.startswith("handoff"):
+    if args.pattern.startswith(("handoff", "scheduler")):
         print(json.dumps(run_handoff_bench(args, load_workload(args.config or 2))))
         return
 
@@ -669,8 +672,9 @@ def run_handoff_bench(args, w):
     clock from the first allocation to the GPU having finished the last copy."""
     import torch
 
-    from distserve_amd import (CacheConfig, ContextStageLLMEngine, DecodingStageLLMEngine, ModelConfig,
-                               ParallelConfig, cabi, create_request, workloads)
+    from distserve_amd import (CacheConfig, ContextStageLLMEngine, DecodingStageFCFSScheduler,
+                               DecodingStageLLMEngine, DecodingStageSchedConfig, ModelConfig, ParallelConfig, cabi,
+                               create_request, workloads)
 
     assert not w.recycles_blocks and w.dec_pp == 1 and w.dec_tp == 1, "handoff patterns run configurations 1-3"
     s = w.shape
@@ -686,7 +690,15 @@ def run_handoff_bench(args, w):
     for i, worker in enumerate(x for row in ctx.workers for x in row):
         worker.k_cache.copy_(workloads.fill_uniform(worker.k_cache.shape, w.seed + i, "cuda"))
         worker.v_cache.copy_(workloads.fill_uniform(worker.v_cache.shape, w.seed + 500 + i, "cuda"))
-    batched = args.pattern == "handoff-batched"
+    batched = args.pattern in ("handoff-batched", "scheduler-batched")
+    sched = None
+    if args.pattern.startswith("scheduler"):
+        # every request of the step is acceptable: the threshold on waiting prompts is off and
+        # the pool holds them all, so the scheduler's work is its decisions, not a refusal
+        sched = DecodingStageFCFSScheduler(
+            DecodingStageSchedConfig("fcfs", len(w.calls), 1 << 30, waiting_block_prop_threshold=1.0),
+            dec.parallel_config, dec.block_manager, dec._migrate_blocks,
+            engine_migrate_blocks_batched_callback=dec._migrate_blocks_batched, batch_migrations=batched)
 
     # where the host time of a hand-off goes: the three steps of _migrate_blocks, timed apart
     spent = {"allocate": 0.0, "migrate_call": 0.0, "release": 0.0}
@@ -720,7 +732,13 @@ def run_handoff_bench(args, w):
             migrating.append(ctx.on_prefill_finished(req))
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        if batched:
+        if sched is not None:
+            for m in migrating:
+                sched.add_request(m)
+            sched.post_process()
+            assert not sched.unaccepted_queue and len(sched.waiting_queue) == len(migrating)
+            sched.waiting_queue.clear()
+        elif batched:
             dec._migrate_blocks_batched(migrating)
         else:
             for m in migrating:
@@ -778,7 +796,8 @@ def run_handoff_bench(args, w):
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u8", "data": "synthetic",
         "config": {"workload": f"{w.name}: {len(w.calls)} requests, {w.total_blocks} blocks",
-                   "pattern": ("BlockManager.allocate_blocks + Worker.migrate_blocks (torch op) + release of the "
+                   "pattern": (("bridge queue -> DecodingStageFCFSScheduler.post_process -> " if sched is not None else "")
+                               + "BlockManager.allocate_blocks + Worker.migrate_blocks (torch op) + release of the "
                                "context blocks, " + ("one migrate call per batch" if batched else "one per request")),
                    "value_counts": "HBM bytes read + written per second of host wall clock (allocation to GPU idle)"},
         "us_per_request": round(ms_per_step * 1e3 / len(w.calls), 2),

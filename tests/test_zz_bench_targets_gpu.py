@@ -124,3 +124,18 @@ def test_swap_line_meets_the_target():
     alone = overlapped["migration_ms_alone"]
     beside = sorted(overlapped["migration_ms_beside_swap_out"] + overlapped["migration_ms_beside_swap_in"])
     assert beside[len(beside) // 2] <= 1.25 * alone, overlapped
+
+
+@pytest.mark.parametrize("pattern", ["handoff", "scheduler", "scheduler-batched"])
+def test_hand_off_lines_are_bit_exact_and_keep_the_workloads_tables(pattern):
+    """The whole hand-off (block allocation, the torch op, release of the context blocks), alone
+    or driven by the decoding scheduler: same bytes, same block tables, and the host work per
+    request stays a fraction of the copy."""
+    line = run_bench("--config", "2", "--pattern", pattern, "--steps", "5", "--warmup", "2")
+    assert line["bit_exact"] is True and line["block_tables_equal_workload"] is True
+    assert line["unit"] == "GB/s" and line["frac_of_hbm_peak"] >= 0.70, line["frac_of_hbm_peak"]
+    assert 0 < line["host_us_per_request"] < line["us_per_request"]
+    # the end stamped after the copy covers it; stamped at the return of the calls it does not
+    assert line["transmission_us_per_request"] > line["transmission_us_per_request_stamped_at_enqueue"]
+    if pattern.startswith("scheduler"):
+        assert "post_process" in line["config"]["pattern"]
