@@ -426,7 +426,7 @@ std::map<SourceKey, Source> g_sources;
 // in the allocation, and the mapping stays until kvm_reset.
 struct Opened {
     int64_t pid, remote_base, size;
-    hipIpcMemHandle_t handle;
+    int64_t serial;   // the exporter's id of the allocation; a new allocation at an old address has another
     char *local_base;
 };
 std::vector<Opened> g_opened;   // guarded by g_mu
@@ -438,8 +438,14 @@ enum {
     kHwCheck = 16,
 };
 static_assert(sizeof(hipIpcMemHandle_t) == 64 && kHwCheck + 1 == KVM_HANDLE_WORDS, "handle layout");
-constexpr int64_t kHandleMagic = 0x4b564d4f56453032LL;  // "KVMOVE02"
+constexpr int64_t kHandleMagic = 0x4b564d4f56453033LL;  // "KVMOVE03"
 constexpr int64_t kHandleHasIpc = 1;                    // flag: words 8..15 hold an exported IPC handle
+// The flags word carries the flags in its low byte and, above it, the runtime's id of the
+// allocation in the exporting process (HIP_POINTER_ATTRIBUTE_BUFFER_ID: every allocation of
+// a process gets a new one).  Together with (pid, base, size) it says whether two handles
+// name the same allocation; the bytes of hipIpcMemHandle_t do not -- two exports of one
+// allocation differ in bytes the runtime leaves unset.
+constexpr int kHandleSerialShift = 8;
 
 int64_t handle_check(const int64_t *h)
 {
@@ -1003,9 +1009,15 @@ int kvm_get_mem_handle(const void *dev_ptr, int64_t nbytes, int64_t *out_handle)
         h[kHwAllocSize] = (int64_t)size;
         if ((int64_t)size < KVM_IPC_MAX_ALLOC_BYTES) {
             hipIpcMemHandle_t ipc;
+            memset(&ipc, 0, sizeof ipc);
             if (hipIpcGetMemHandle(&ipc, base) == hipSuccess) {
                 memcpy(&h[kHwIpc], &ipc, sizeof ipc);
                 h[kHwFlags] |= kHandleHasIpc;
+                unsigned long long id = 0;
+                if (hipPointerGetAttribute(&id, HIP_POINTER_ATTRIBUTE_BUFFER_ID, base) == hipSuccess)
+                    h[kHwFlags] |= (int64_t)((id & 0x7fffffffffffffull) << kHandleSerialShift);
+                else
+                    (void)hipGetLastError();   // no id: (pid, base, size) alone names the allocation
             } else {
                 (void)hipGetLastError();   // stays a handle for this process only
             }
@@ -1050,10 +1062,15 @@ static int open_handle(const int64_t *h, const char *what, const char **ptr, int
                     (long long)h[kHwAllocSize]);
     hipIpcMemHandle_t ipc;
     memcpy(&ipc, &h[kHwIpc], sizeof ipc);
+    const int64_t serial = (int64_t)((uint64_t)h[kHwFlags] >> kHandleSerialShift);
     for (size_t i = 0; i < g_opened.size(); ++i) {
         Opened &o = g_opened[i];
         if (o.pid != h[kHwPid] || o.remote_base != h[kHwAllocBase]) continue;
-        if (o.size == h[kHwAllocSize] && memcmp(&o.handle, &ipc, sizeof ipc) == 0) {
+        if (o.serial == serial) {
+            if (o.size != h[kHwAllocSize])
+                return fail(KVM_EHANDLE, "%s handle of process %lld says its allocation holds %lld bytes, the same "
+                            "allocation is open with %lld", what, (long long)h[kHwPid], (long long)h[kHwAllocSize],
+                            (long long)o.size);
             *ptr = o.local_base + off;
             *map = o.local_base;
             return KVM_OK;
@@ -1082,7 +1099,7 @@ static int open_handle(const int64_t *h, const char *what, const char **ptr, int
         return fail(KVM_EHANDLE, "%s handle of process %lld says its allocation holds %lld bytes, the mapping holds %llu",
                     what, (long long)h[kHwPid], (long long)h[kHwAllocSize], (unsigned long long)mapped);
     }
-    g_opened.push_back(Opened{h[kHwPid], h[kHwAllocBase], h[kHwAllocSize], ipc, (char *)local});
+    g_opened.push_back(Opened{h[kHwPid], h[kHwAllocBase], h[kHwAllocSize], serial, (char *)local});
     *ptr = (char *)local + off;
     *map = (char *)local;
     return KVM_OK;

@@ -97,6 +97,9 @@ int kvm_get_mem_handle(const void *dev_ptr, int64_t nbytes, int64_t *out_handle)
  * (distserve/config.py:57-63).  Registering the same rank again replaces the binding.
  * Handles made by another process are opened here (hipIpcOpenMemHandle, once per
  * allocation and process, however many pools lie in it) and stay mapped until kvm_reset.
+ * A handle carries the exporting runtime's id of its allocation: when the exporter has
+ * freed its pools and allocated new ones, handles exported afterwards replace the stale
+ * mapping (and drop the pools bound through it) even where an address recurs.
  * ctx_instance (no counterpart in the reference, whose decoding worker serves a single
  * context instance) keeps the pools of several context instances apart in one process:
  * bindings are keyed by (ctx_instance, pp_rank, tp_rank), and a migrate call reads the

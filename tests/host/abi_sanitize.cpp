@@ -128,7 +128,7 @@ int main()
     EXPECT(kvm_register_mem_handle(nullptr, h, 4, 4, pc, pc, 0) == KVM_EINVAL);
     EXPECT(kvm_register_mem_handle(h, h, 4, 4, nullptr, pc, 0) == KVM_EINVAL);
     EXPECT(kvm_register_mem_handle(h, h, 4, 4, pc, bad_pc, 0) == KVM_EINVAL);
-    h[0] = 0x4b564d4f56453032LL; h[1] = 1; h[2] = 0; h[3] = 4096; h[4] = 64;   // plausible but forged: checksum missing
+    h[0] = 0x4b564d4f56453033LL; h[1] = 1; h[2] = 0; h[3] = 4096; h[4] = 64;   // plausible but forged: checksum missing
     EXPECT(kvm_register_mem_handle(h, h, 4, 4, pc, pc, 0) == KVM_EHANDLE);
     EXPECT(std::strstr(kvm_last_error(), "not a kvmove memory handle") != nullptr);
     // well-formed handles of another process (pid 1), with the checksum word as the library computes it

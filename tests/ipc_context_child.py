@@ -10,6 +10,8 @@ memory handles ``[pp][tp] = (k, v)`` and the block tables.  Commands afterwards:
 ``{"cmd": "verify"}``             are the pools still what the seed says?  -> ``{"unchanged": bool}``
 ``{"cmd": "release", "id": n}``   free request n's blocks                   -> ``{"released": n}``
 ``{"cmd": "big_handle"}``         handle of a pool in an allocation of 2 GiB and more -> ``{"handle": [...]}``
+``{"cmd": "reallocate", "seed": s}``  free every pool, hand the memory back to the runtime, allocate the pools
+                                  again filled from seed s -> ``{"handles": ..., "tables": ...}``
 ``{"cmd": "exit"}``
 """
 import json
@@ -72,6 +74,22 @@ def main() -> None:
             big = torch.empty((2 << 30) + (4 << 20), dtype=torch.uint8, device="cuda")
             piece = big[1 << 30:(1 << 30) + (1 << 20)]
             print(json.dumps({"handle": torch.ops.block_migration_ops.get_ipc_mem_handle(piece)}), flush=True)
+        elif msg["cmd"] == "reallocate":
+            for w in workers:
+                w.k_cache = w.v_cache = w.k_swap = w.v_swap = None
+            torch.cuda.synchronize()
+            torch.cuda.empty_cache()
+            spec["seed"] = msg["seed"]
+            ctx._init_kvcache(spec["blocks"], 0)
+            for i, w in enumerate(workers):
+                w.k_cache.copy_(workloads.fill_uniform(w.k_cache.shape, pool_seed(spec["seed"], i, False)))
+                w.v_cache.copy_(workloads.fill_uniform(w.v_cache.shape, pool_seed(spec["seed"], i, True)))
+            torch.cuda.synchronize()
+            tables = {}
+            for rid, prompt_len in enumerate(spec["prompts"]):
+                ctx.block_manager.allocate_blocks(create_request(prompt_len, rid))
+                tables[rid] = list(ctx.block_manager.get_block_table(rid))
+            print(json.dumps({"handles": ctx.kv_cache_mem_handles, "tables": tables}), flush=True)
         elif msg["cmd"] == "exit":
             break
     del big

@@ -186,6 +186,67 @@ def test_context_instance_in_another_process_tp2pp2_to_tp4_every_rank_against_or
             kvm.register_mem_handle(lie, lie, 8, 8, [1, 0, 1, 0], [1, 0, 1, 0])
         assert e.value.code == kvm.KVM_EHANDLE and "the mapping holds" in str(e.value)
         assert kvm.opened_handles() == 0
+        # ... and while the allocation is open under its true size, it unbinds nothing
+        dec.register_kvcache_mem_handles(ctx_config, handles)
+        # one mapping per allocation of the other process, however many pools lie in it and
+        # however often they are registered
+        allocations = {(h[1], h[5]) for row in handles for pair in row for h in pair}
+        assert kvm.opened_handles() == len(allocations)
+        with pytest.raises(kvm.KvmError) as e:
+            kvm.register_mem_handle(lie, lie, 8, 8, [1, 0, 1, 0], [1, 0, 1, 0], ctx_instance=9)
+        assert e.value.code == kvm.KVM_EHANDLE and "is open with" in str(e.value)
+        assert kvm.opened_handles() == len(allocations)
+        # binding the same pools a second time, as another context instance, leaves the first
+        # binding alone: both resolve through the mapping that is already open
+        k00, v00 = handles[0][0]
+        kvm.register_mem_handle(k00, v00, 8, 8, [2, 0, 2, 0], [4, 0, 1, 0], ctx_instance=7)
+        assert kvm.opened_handles() == len(allocations)
+        dw = dec.workers[0][0]
+        dw.migrate_blocks(tables[0], ctx_config, list(range(len(tables[0]))))     # instance 0 is still bound
+        torch.cuda.synchronize()
+    finally:
+        ctx.close()
+        kvm.reset()
+    assert ctx.proc.returncode == 0, open(ctx.log_path).read()[-3000:]
+
+
+def test_pools_reallocated_by_the_other_process_replace_their_stale_mappings(kvm, tmp_path):
+    """The context process frees its pools and allocates them again (the runtime may hand out
+    the same addresses): handles exported afterwards name other allocations, and registering
+    them must not resolve through the mappings of the freed ones."""
+    kvm.reset()
+    spec = dict(SPEC, seed=520, prompts=[48, 80], busy_blocks=0)
+    ctx = ContextProcess(spec, str(tmp_path / "context_process.log"))
+    try:
+        model = ModelConfig.from_kv_shape(num_layers=8, num_heads=8, head_dim=64, num_kv_heads=8)
+        ctx_config = ParallelConfig(2, 0, 2, 0)
+        dec = DecodingStageLLMEngine(model, ParallelConfig(1, 0, 1, 0), CacheConfig(16, 64))
+        dec._init_kvcache(32, 0)
+        dw = dec.workers[0][0]
+        g = oracle.Geom(8, 8, 16, 64, 2, 2, 2, 1, 1)
+        handles, tables, seen = ctx.hello["handles"], ctx.hello["tables"], []
+        for generation, seed in enumerate((520, 521, 522)):
+            if generation:
+                answer = ctx.ask({"cmd": "reallocate", "seed": seed}, timeout=120)
+                handles, tables = answer["handles"], answer["tables"]
+            seen.append({(h[5], h[7] >> 8) for row in handles for pair in row for h in pair})
+            dec.register_kvcache_mem_handles(ctx_config, handles)     # no reset in between
+            src_k, src_v = child_sources(dict(spec, seed=seed))
+            dw.k_cache.view(torch.int16).fill_(0x7C01)
+            dw.v_cache.view(torch.int16).fill_(0x7C01)
+            want_k, want_v = canary_pool(dw.k_cache.shape), canary_pool(dw.v_cache.shape)
+            for rid in ("0", "1"):
+                di = list(range(3 + 8 * int(rid), 3 + 8 * int(rid) + len(tables[rid])))
+                dw.migrate_blocks(tables[rid], ctx_config, di)
+                oracle.migrate_c(g, src_k, tables[rid], di, want_k)
+                oracle.migrate_c(g, src_v, tables[rid], di, want_v)
+            torch.cuda.synchronize()
+            assert same_bits(dw.k_cache.cpu(), want_k) and same_bits(dw.v_cache.cpu(), want_v), generation
+            assert kvm.opened_handles() <= sum(len({base for base, _ in s}) for s in seen)
+        reused = [len({b for b, _ in seen[i]} & {b for b, _ in seen[i + 1]}) for i in range(2)]
+        print("addresses handed out again from one generation to the next:", reused)
+        # every generation's allocations carried ids of their own
+        assert not (seen[0] & seen[1]) and not (seen[1] & seen[2])
     finally:
         ctx.close()
         kvm.reset()
