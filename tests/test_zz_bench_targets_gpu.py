@@ -103,13 +103,13 @@ def test_configurations_3_and_4_reach_what_the_plainest_kernel_reaches_on_their_
     assert len(per_request) == 3 and len(long_launch) == 3, rows
     assert all(3000 < v < 8000 for v in per_request + long_launch), rows
     configs = default_line()["configs"]
-    assert configs["cfg4"]["GBps"] >= 0.93 * max(per_request), (configs["cfg4"]["GBps"], per_request)
-    assert configs["cfg4_batched"]["GBps"] >= 0.93 * max(long_launch), (configs["cfg4_batched"]["GBps"], long_launch)
+    assert configs["cfg4"]["GBps"] >= 0.90 * max(per_request), (configs["cfg4"]["GBps"], per_request)
+    assert configs["cfg4_batched"]["GBps"] >= 0.90 * max(long_launch), (configs["cfg4_batched"]["GBps"], long_launch)
     # configuration 3's geometry: whole blocks, 80 KiB pieces of two pools side by side
     rows = [r for r in table if r[0] == "13B 2 x 80 KiB" and r[1] == "random" and r[2] == "random"]
     per_request = [float(r[-1]) for r in rows if r[3] == "72"]
     assert len(per_request) == 3, rows
-    assert configs["cfg3"]["GBps"] >= 0.93 * max(per_request), (configs["cfg3"]["GBps"], per_request)
+    assert configs["cfg3"]["GBps"] >= 0.90 * max(per_request), (configs["cfg3"]["GBps"], per_request)
 
 
 def test_swap_line_meets_the_target():
