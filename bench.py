@@ -42,11 +42,14 @@ def parse_args():
                     help="configuration 4 only: context tensor-parallel size. 2 is the configuration itself (8 KiB runs "
                          "at a 16 KiB source stride); 4 moves the same bytes from dense source pools, for comparison")
     ap.add_argument("--pattern", default="request",
-                    choices=["request", "batch", "handoff", "handoff-batched", "scheduler", "scheduler-batched"],
+                    choices=["request", "batch", "handoff", "handoff-batched", "scheduler", "scheduler-batched", "ipc"],
                     help="handoff*: the same requests through Worker / BlockManager / the migration handoff "
                          "(torch ops, block allocation and release included), one call per request or one per batch; "
                          "scheduler*: the same, with the decoding scheduler's post_process deciding acceptance "
-                         "(bridge queue -> scheduler -> engine -> op), batch_migrations off or on")
+                         "(bridge queue -> scheduler -> engine -> op), batch_migrations off or on; "
+                         "ipc: configuration 2's shape with the context pools in ANOTHER process (memory handles "
+                         "over a pipe, hipIpc mapping), against the same pools in this process")
+    ap.add_argument("--ipc-child", action="store_true", help=argparse.SUPPRESS)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-verify", action="store_true")
     ap.add_argument("--opt", action="append", default=[], help="kvmove tuning option name=value")
@@ -333,10 +336,17 @@ def compact(d: dict) -> dict:
 
 def main():
     args = parse_args()
+    if args.ipc_child:
+        run_ipc_child()
+        return
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (source and destination pools share one HBM; "
               "there is no sharding or collective on this path); run with --gpus 1", file=sys.stderr)
         sys.exit(2)
+
+    if args.pattern == "ipc":
+        print(json.dumps(run_ipc_bench(args)))    # starts its child before this process touches the GPU
+        return
 
     import torch
 
@@ -662,6 +672,140 @@ def swap_cpu_baseline(w, sample_blocks=256, budget_s=10.0):
                        f"{len(w.out_gpu_ids)} blocks out and back, pools compacted to the sample, {passes} passes in "
                        f"{dt:.1f} s; GB/s counts bytes copied, like the link figure"),
             "host_cpu_count": os.cpu_count()}
+
+
+IPC_POOL_BLOCKS = 448    # 1.75 GiB per pool at the LLaMA-2-7B shape: pools that cross a process boundary stay under 2 GiB
+IPC_SEED = 77
+
+
+def run_ipc_child():
+    """The context instance of `--pattern ipc`, in a process of its own: makes the K and V
+    pools the first line on stdin describes, prints its pid and their memory handles as one
+    JSON line, and keeps the pools alive until stdin says anything more or closes."""
+    spec = json.loads(sys.stdin.readline())
+    import torch
+
+    from distserve_amd import cabi, workloads
+
+    torch.cuda.set_device(0)
+    k = workloads.fill_uniform(tuple(spec["shape"]), spec["seed"], "cuda")
+    v = workloads.fill_uniform(tuple(spec["shape"]), spec["seed"] + 500, "cuda")
+    torch.cuda.synchronize()
+    nbytes = k.numel() * k.element_size()
+    print(json.dumps({"pid": os.getpid(), "k": cabi.get_mem_handle(k.data_ptr(), nbytes),
+                      "v": cabi.get_mem_handle(v.data_ptr(), nbytes)}), flush=True)
+    sys.stdin.readline()
+
+
+def run_ipc_bench(args):
+    """Migration out of pools that another process owns.  The child (this file again, started
+    before this process touches the GPU) holds the context pools and sends their handles; this
+    process binds them as context instance 1 and, for comparison, identical pools of its own
+    as instance 2, then times the same 7 calls of 64 blocks out of each, alternating."""
+    import subprocess
+    import threading
+
+    child = subprocess.Popen([sys.executable, "-u", os.path.abspath(__file__), "--ipc-child"], stdin=subprocess.PIPE,
+                             stdout=subprocess.PIPE, text=True, cwd=os.path.dirname(os.path.abspath(__file__)))
+    try:
+        from distserve_amd import workloads as wl
+
+        s = wl.config2().shape
+        shape = (IPC_POOL_BLOCKS, s.num_layers, s.num_kv_heads, s.block_size, s.head_dim)
+        child.stdin.write(json.dumps({"shape": shape, "seed": IPC_SEED}) + "\n")
+        child.stdin.flush()
+        answer = {}
+        reader = threading.Thread(target=lambda: answer.update(line=child.stdout.readline()), daemon=True)
+        reader.start()
+        reader.join(timeout=400)          # the child's first import of torch can take minutes on a fresh box
+        if not answer.get("line"):
+            raise RuntimeError("the context process did not send its handles")
+        hello = json.loads(answer["line"])
+
+        import torch
+
+        from distserve_amd import cabi
+
+        if not torch.cuda.is_available():
+            raise RuntimeError("no GPU visible; the KV movement path has no CPU fallback")
+        for kv in args.opt:
+            name, value = kv.split("=")
+            cabi.set_option(name, int(value))
+        torch.cuda.set_device(0)
+        stream = torch.cuda.current_stream()
+        cabi.reset()
+        pc = [1, 0, 1, 0]
+        cabi.register_mem_handle(hello["k"], hello["v"], s.num_layers, s.num_kv_heads, pc, pc, ctx_instance=1)
+        opened = cabi.opened_handles()
+        own_k = wl.fill_uniform(shape, IPC_SEED, "cuda")
+        own_v = wl.fill_uniform(shape, IPC_SEED + 500, "cuda")
+        nbytes = own_k.numel() * own_k.element_size()
+        cabi.register_source(1, 1, 0, 0, s.num_layers, s.num_kv_heads, own_k.data_ptr(), own_v.data_ptr(), nbytes,
+                             ctx_instance=2)
+        dst_k, dst_v = wl.fill_canary(shape, "cuda"), wl.fill_canary(shape, "cuda")
+        g = torch.Generator().manual_seed(IPC_SEED)
+        src_order = torch.randperm(IPC_POOL_BLOCKS, generator=g).tolist()
+        dst_order = torch.randperm(IPC_POOL_BLOCKS, generator=g).tolist()
+        calls = [(cabi.index_array(src_order[i:i + 64]), cabi.index_array(dst_order[i:i + 64]))
+                 for i in range(0, IPC_POOL_BLOCKS, 64)]
+        geoms = {name: cabi.geom(s.num_layers, s.num_kv_heads, s.block_size, s.head_dim, s.dtype_bytes, ctx_instance=inst)
+                 for name, inst in (("other_process", 1), ("this_process", 2))}
+
+        def step(geom):
+            for ci, di in calls:
+                cabi.migrate(geom, ci, di, dst_k.data_ptr(), dst_v.data_ptr(), IPC_POOL_BLOCKS, stream.cuda_stream)
+
+        def timed(geom, steps):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record(stream)
+            for _ in range(steps):
+                step(geom)
+            b.record(stream)
+            torch.cuda.synchronize()
+            return a.elapsed_time(b) / steps
+
+        exact = {}
+        for name, geom in geoms.items():
+            dst_k.view(torch.int16).fill_(0x7C01)
+            dst_v.view(torch.int16).fill_(0x7C01)
+            for _ in range(args.warmup):
+                step(geom)
+            torch.cuda.synchronize()
+            # every block of the pools is a destination once: the whole pools must be the gather
+            si, di = torch.tensor(src_order, device="cuda"), torch.tensor(dst_order, device="cuda")
+            exact[name] = bool(torch.equal(dst_k[di].view(torch.int16), own_k[si].view(torch.int16))
+                               and torch.equal(dst_v[di].view(torch.int16), own_v[si].view(torch.int16)))
+        ms = {name: [] for name in geoms}
+        for _ in range(5):                       # alternating, so that drift hits both alike
+            for name, geom in geoms.items():
+                ms[name].append(timed(geom, max(1, args.steps // 5)))
+        hbm_bytes = 4 * nbytes                   # both pools, read once and written once
+        med = {name: sorted(v)[len(v) // 2] for name, v in ms.items()}
+        gbps = {name: hbm_bytes / (m * 1e-3) / 1e9 for name, m in med.items()}
+        cabi.reset()
+        return {
+            "metric": "KV migration GB/s out of another process's pools (hipIpc mapping), LLaMA-2-7B shape",
+            "value": round(gbps["other_process"], 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+            "warmup": args.warmup, "ms_per_step": round(med["other_process"], 4), "higher_is_better": True,
+            "scaling": "weak", "vs_baseline": None, "dtype": "u8", "data": "synthetic",
+            "config": {"workload": f"cfg2 shape, {IPC_POOL_BLOCKS}-block pools ({nbytes >> 20} MiB each, below the 2 GiB "
+                                   f"export limit), {len(calls)} calls of 64 blocks, every block moved once, seed {IPC_SEED}",
+                       "pattern": "context pools in a child process, handles over a pipe; the same calls out of "
+                                  "identical pools of this process, alternating, median of 5 rounds each"},
+            "frac_of_hbm_peak": round(gbps["other_process"] / HBM_PEAK_GBPS, 4),
+            "this_process_GBps": round(gbps["this_process"], 2),
+            "other_over_this_process": round(gbps["other_process"] / gbps["this_process"], 4),
+            "us_per_call": {name: round(m * 1e3 / len(calls), 2) for name, m in med.items()},
+            "context_process_pid": hello["pid"], "this_pid": os.getpid(), "mappings_opened": opened,
+            "bit_exact": all(exact.values()), "bit_exact_by_source": exact,
+        }
+    finally:
+        try:
+            child.stdin.write("\n")
+            child.stdin.flush()
+            child.wait(timeout=60)
+        except Exception:
+            child.kill()
 
 
 def run_handoff_bench(args, w):

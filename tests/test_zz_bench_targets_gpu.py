@@ -139,3 +139,13 @@ def test_hand_off_lines_are_bit_exact_and_keep_the_workloads_tables(pattern):
     assert line["transmission_us_per_request"] > line["transmission_us_per_request_stamped_at_enqueue"]
     if pattern.startswith("scheduler"):
         assert "post_process" in line["config"]["pattern"]
+
+
+def test_migration_out_of_another_process_runs_at_the_speed_of_local_pools():
+    """`--pattern ipc`: the context pools live in a child process and are read through their
+    hipIpc mapping; the same calls out of identical local pools are timed beside them."""
+    line = run_bench("--pattern", "ipc", "--steps", "10", "--warmup", "2", timeout=600)
+    assert line["bit_exact"] is True and line["bit_exact_by_source"] == {"other_process": True, "this_process": True}
+    assert line["context_process_pid"] != line["this_pid"] and line["mappings_opened"] == 2
+    assert line["frac_of_hbm_peak"] >= 0.70
+    assert line["other_over_this_process"] >= 0.90, line
