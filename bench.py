@@ -408,6 +408,17 @@ def main():
                                "pattern": "64-block calls out of 1.75 GiB pools held by a child process (hipIpc mapping)"}
     except Exception as e:      # noqa: BLE001 - reported, not hidden
         configs["cfg2_ipc"] = {"error": f"{type(e).__name__}: {e}"}
+    # the whole hand-off at configuration 2 (block allocation, the torch op, release of the context
+    # blocks), driven by the decoding scheduler, with the transmission time the lifetime events give
+    import copy
+
+    hand = copy.copy(args)
+    hand.pattern, hand.no_verify = "scheduler", not verify_result
+    h = run_handoff_bench(hand, load_workload(2))
+    configs["cfg2_handoff"] = {k: h[k] for k in (
+        "us_per_request", "host_us_per_request", "transmission_us_per_request",
+        "transmission_us_per_request_stamped_at_enqueue", "frac_of_hbm_peak", "block_tables_equal_workload", "bit_exact")}
+    configs["cfg2_handoff"].update(GBps=h["value"], pattern=h["config"]["pattern"])
     out["configs"] = configs
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(w2)

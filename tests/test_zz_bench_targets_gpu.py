@@ -74,7 +74,11 @@ def test_migration_line_meets_the_contract_and_the_target():
     assert 0 < line["host_call_us"] < 100                     # one call on an idle stream: microseconds
     # every other configuration rides along in the same line
     configs = line["configs"]
-    assert sorted(configs) == ["cfg1", "cfg2_batched", "cfg2_ipc", "cfg3", "cfg3_batched", "cfg4", "cfg4_batched", "cfg5"]
+    assert sorted(configs) == ["cfg1", "cfg2_batched", "cfg2_handoff", "cfg2_ipc", "cfg3", "cfg3_batched", "cfg4",
+                               "cfg4_batched", "cfg5"]
+    hand = configs["cfg2_handoff"]
+    assert hand["bit_exact"] is True and hand["block_tables_equal_workload"] is True and hand["frac_of_hbm_peak"] >= 0.70
+    assert hand["transmission_us_per_request"] > hand["transmission_us_per_request_stamped_at_enqueue"] > 0
     assert configs["cfg2_ipc"].get("bit_exact") is True and configs["cfg2_ipc"]["other_over_this_process"] >= 0.90, \
         configs["cfg2_ipc"]
     for name in ("cfg1", "cfg2_batched", "cfg3", "cfg3_batched", "cfg4", "cfg4_batched"):
