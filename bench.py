@@ -41,6 +41,9 @@ def parse_args():
     ap.add_argument("--ctx-tp", type=int, default=0,
                     help="configuration 4 only: context tensor-parallel size. 2 is the configuration itself (8 KiB runs "
                          "at a 16 KiB source stride); 4 moves the same bytes from dense source pools, for comparison")
+    ap.add_argument("--fresh-pools", action="store_true",
+                    help="configurations 2-4, a comparison: block managers that have just started (free lists "
+                         "0..n-1, a request's blocks are neighbours) instead of pools in service (shuffled lists)")
     ap.add_argument("--pattern", default="request",
                     choices=["request", "batch", "handoff", "handoff-batched", "scheduler", "scheduler-batched", "ipc"],
                     help="handoff*: the same requests through Worker / BlockManager / the migration handoff "
@@ -171,11 +174,13 @@ def cpu_baseline(w, budget_s=12.0):
     }
 
 
-def load_workload(config: int, ctx_tp=None):
+def load_workload(config: int, ctx_tp=None, fresh_pools=False):
     from distserve_amd import workloads
 
-    if config == 4 and ctx_tp:
-        return workloads.config4(ctx_tp=ctx_tp)
+    if config == 4 and (ctx_tp or fresh_pools):
+        return workloads.config4(ctx_tp=ctx_tp or 2, fresh_pools=fresh_pools)
+    if config in (2, 3) and fresh_pools:
+        return {2: workloads.config2, 3: workloads.config3}[config](fresh_pools=True)
     return {1: workloads.config1, 2: workloads.config2, 3: workloads.config3, 4: workloads.config4}[config]()
 
 
@@ -199,14 +204,14 @@ def host_call_cost_us(cabi, geom, w, dst_k, dst_v, stream, calls=64):
 
 
 def bench_migrate(config: int, pattern: str, steps: int, warmup: int, verify_result: bool = True,
-                  calibrate_copy: bool = False, ctx_tp=None):
+                  calibrate_copy: bool = False, ctx_tp=None, fresh_pools=False):
     """Times one migration workload; returns (record, workload).  Pools are made, timed and
     freed inside."""
     import torch
 
     from distserve_amd import cabi, workloads
 
-    w = load_workload(config, ctx_tp)
+    w = load_workload(config, ctx_tp, fresh_pools)
     torch.cuda.set_device(0)
     stream = torch.cuda.current_stream()
     s = w.shape
@@ -273,7 +278,7 @@ def bench_migrate(config: int, pattern: str, steps: int, warmup: int, verify_res
     copy_ceiling = time_plain_copy(cabi, stream) if calibrate_copy else None
 
     tuning = {k: cabi.get_option(k) for k in ("tile_bytes", "threads", "unroll", "nt_load", "nt_store")}
-    traffic, traffic_source = measured_traffic(config if not ctx_tp else 0, bytes_per_launch)
+    traffic, traffic_source = measured_traffic(config if not (ctx_tp or fresh_pools) else 0, bytes_per_launch)
     cache_resident = 2 * hbm_bytes <= INFINITY_CACHE_BYTES
     out = {
         "metric": "KV migration GB/s (% of HBM peak) + us/request at LLaMA-2-7B shape" if config == 2
@@ -381,7 +386,7 @@ def main():
     if args.config:
         # one configuration, nothing else launched: the command the kernel profiles are taken with
         out, w = bench_migrate(args.config, args.pattern, args.steps, args.warmup, verify_result,
-                               args.calibrate_copy, args.ctx_tp)
+                               args.calibrate_copy, args.ctx_tp, args.fresh_pools)
         if not args.no_cpu_baseline:
             out["cpu_baseline"] = cpu_baseline(w)
         print(json.dumps(out))

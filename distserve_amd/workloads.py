@@ -90,10 +90,13 @@ def _lengths(g: torch.Generator, n: int, lo: int, hi: int) -> List[int]:
 
 
 def _disjoint_calls(g: torch.Generator, lengths: List[int], block_size: int, src_blocks: int,
-                    dst_blocks: int) -> List[MigrateCall]:
-    """Per-request slices of two independent random permutations: non-contiguous and disjoint."""
+                    dst_blocks: int, fresh: bool = False) -> List[MigrateCall]:
+    """Per-request slices of two independent random permutations: non-contiguous and disjoint.
+    ``fresh``: slices of ``0 .. n-1`` instead, what block managers hand out when they start."""
     src_perm = torch.randperm(src_blocks, generator=g).tolist()
     dst_perm = torch.randperm(dst_blocks, generator=g).tolist()
+    if fresh:
+        src_perm, dst_perm = list(range(src_blocks)), list(range(dst_blocks))
     calls, at = [], 0
     for rid, length in enumerate(lengths):
         n = blocks_for(length, block_size)
@@ -105,10 +108,11 @@ def _disjoint_calls(g: torch.Generator, lengths: List[int], block_size: int, src
 
 class _ShuffledFifo:
     """Free list with the block manager's discipline (take from the head, give back at the
-    tail) but a shuffled initial order, as a pool looks after it has run for a while."""
+    tail) but a shuffled initial order, as a pool looks after it has run for a while.
+    ``fresh``: the order a block manager starts with, ``0 .. n-1``."""
 
-    def __init__(self, n: int, g: torch.Generator):
-        self.free = torch.randperm(n, generator=g).tolist()
+    def __init__(self, n: int, g: torch.Generator, fresh: bool = False):
+        self.free = list(range(n)) if fresh else torch.randperm(n, generator=g).tolist()
 
     def take(self, n: int) -> List[int]:
         assert len(self.free) >= n
@@ -120,11 +124,11 @@ class _ShuffledFifo:
 
 
 def _recycled_calls(g: torch.Generator, lengths: List[int], block_size: int, src_blocks: int,
-                    dst_blocks: int) -> List[MigrateCall]:
+                    dst_blocks: int, fresh: bool = False) -> List[MigrateCall]:
     """Sequential hand-offs through pools smaller than the batch: the context side frees a
     request's blocks right after its migration (as the engine does), the decoding side
     frees its oldest requests when it runs short."""
-    src, dst = _ShuffledFifo(src_blocks, g), _ShuffledFifo(dst_blocks, g)
+    src, dst = _ShuffledFifo(src_blocks, g, fresh), _ShuffledFifo(dst_blocks, g, fresh)
     resident: List[List[int]] = []
     calls = []
     for rid, length in enumerate(lengths):
@@ -153,36 +157,45 @@ def config1(seed: int = 1) -> MigrateWorkload:
     return w
 
 
-def config2(seed: int = 2, num_requests: int = 16, pool_blocks: int = 4096) -> MigrateWorkload:
+def config2(seed: int = 2, num_requests: int = 16, pool_blocks: int = 4096, fresh_pools: bool = False) -> MigrateWorkload:
     """LLaMA-2-7B KV shape, 16 requests of 64..2048 prompt tokens, TP1 -> TP1."""
     g = torch.Generator().manual_seed(seed)
     shape = KvShape(32, 32, 128)
     w = MigrateWorkload("cfg2-llama2-7b", shape, 1, 1, 1, 1, 0, 0, pool_blocks, pool_blocks, seed)
-    w.calls = _disjoint_calls(g, _lengths(g, num_requests, 64, 2048), 16, pool_blocks, pool_blocks)
+    w.calls = _disjoint_calls(g, _lengths(g, num_requests, 64, 2048), 16, pool_blocks, pool_blocks, fresh_pools)
+    if fresh_pools:
+        w.name += "-fresh-pools"
     return w
 
 
-def config3(seed: int = 3, num_requests: int = 32) -> MigrateWorkload:
+def config3(seed: int = 3, num_requests: int = 32, fresh_pools: bool = False) -> MigrateWorkload:
     """OPT-13B KV shape, context TP2 -> decoding TP1: two 20-head pools merge into one."""
     g = torch.Generator().manual_seed(seed)
     shape = KvShape(40, 40, 128)
     w = MigrateWorkload("cfg3-opt-13b-tp2to1", shape, 1, 2, 1, 1, 0, 0, 2048, 4096, seed)
-    w.calls = _disjoint_calls(g, _lengths(g, num_requests, 128, 1024), 16, 2048, 4096)
+    w.calls = _disjoint_calls(g, _lengths(g, num_requests, 128, 1024), 16, 2048, 4096, fresh_pools)
+    if fresh_pools:
+        w.name += "-fresh-pools"
     return w
 
 
-def config4(seed: int = 4, num_requests: int = 24, ctx_tp: int = 2) -> MigrateWorkload:
+def config4(seed: int = 4, num_requests: int = 24, ctx_tp: int = 2, fresh_pools: bool = False) -> MigrateWorkload:
     """LLaMA-2-70B GQA KV shape, context TP2/PP2 -> decoding TP4 rank 1 (2 of 8 KV heads,
     all 80 layers).  The batch needs more blocks than either pool holds, so the calls
     recycle block ids.  ``ctx_tp=4`` is a comparison layout, not the configuration: the same
     block tables and the same bytes, from context pools that hold exactly the two heads
-    the decoding rank wants, so the sources are read densely."""
+    the decoding rank wants, so the sources are read densely.  ``fresh_pools`` is another
+    comparison: the same requests through block managers that have just started, whose free
+    lists are still ``0 .. n-1``, so that a request's blocks are neighbours in both pools
+    (the configuration itself starts from shuffled lists, the state of a pool in service)."""
     g = torch.Generator().manual_seed(seed)
     shape = KvShape(80, 8, 128)
     name = "cfg4-llama2-70b-tp2pp2to-tp4r1" if ctx_tp == 2 else f"cfg4-variant-tp{ctx_tp}pp2to-tp4r1"
+    if fresh_pools:
+        name += "-fresh-pools"
     w = MigrateWorkload(name, shape, 2, ctx_tp, 1, 4, 0, 1, 1024, 2048, seed,
                         recycles_blocks=True)
-    w.calls = _recycled_calls(g, _lengths(g, num_requests, 256, 4096), 16, 1024, 2048)
+    w.calls = _recycled_calls(g, _lengths(g, num_requests, 256, 4096), 16, 1024, 2048, fresh_pools)
     return w
 
 

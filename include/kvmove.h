@@ -167,7 +167,9 @@ int kvm_copy_plain(void *dst, const void *src, int64_t nbytes, void *stream);
  *   "unroll"         16-byte vectors in flight per lane: 1, 2, 4, 8 or 16
  *   "wave_contig"    1 = a wave's vectors are adjacent in memory, 0 = one pass apart
  *   "lds_pad"        bytes of LDS requested per workgroup only to limit occupancy (0..65536)
- *   "xcd_map"        how workgroup ids map to work: 0 = in order, 1 (default) = each XCD walks
+ *   "xcd_map"        how workgroup ids map to work: 0 = in order, 1 (default) = chosen per call:
+ *                    in order when at least half of the call's context blocks follow their
+ *                    predecessor in the list directly (neighbouring blocks), else each XCD walks
  *                    contiguous chunks (an eighth of a block when that is >= 256 KiB, else an
  *                    eighth of the launch), 2 = always an eighth of the launch, 3 = always an
  *                    eighth of a block

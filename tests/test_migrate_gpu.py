@@ -550,3 +550,27 @@ def test_a_pool_that_claims_more_than_its_allocation_is_refused_on_the_host(kvm)
     torch.cuda.synchronize()
     assert same_bits(dst_k[3].cpu(), src_k[1].cpu())
     kvm.reset()
+
+
+@pytest.mark.parametrize("cpp,ctp,dpp,dtp,q,u", [(1, 1, 1, 1, 0, 0), (2, 2, 1, 4, 0, 1), (1, 2, 1, 1, 0, 0)])
+@pytest.mark.parametrize("lists", ["neighbours", "runs", "scattered", "descending"])
+def test_lists_of_neighbouring_and_of_scattered_blocks_copy_the_same_way(kvm, cpp, ctp, dpp, dtp, q, u, lists):
+    """The order in which a launch's workgroups take the work is chosen from the context block
+    list (in order for mostly neighbouring blocks, per-XCD chunks for scattered ones); the bytes
+    copied must not know about it.  Launches large enough for the chunks to differ from the
+    plain order: 40 blocks of 64-128 tiles each."""
+    import random
+
+    g = oracle.Geom(8, 8, 16, 64, 2, cpp, ctp, dpp, dtp, q, u)
+    rng = random.Random(hash((cpp, ctp, dtp, lists)) & 0xFFFF)
+    nb_src, nb_dst, n = 48, 64, 40
+    if lists == "neighbours":
+        ci = list(range(5, 5 + n))                               # one run: ids in order
+    elif lists == "runs":
+        ci = list(range(30, 44)) + list(range(0, 13)) + list(range(17, 30))   # three runs: still mostly neighbours
+    elif lists == "descending":
+        ci = list(range(n + 3, 3, -1))                           # adjacent the wrong way round: not neighbours
+    else:
+        ci = rng.sample(range(nb_src), n)
+    di = rng.sample(range(nb_dst), n)
+    check_case(kvm, g, nb_src, nb_dst, ci, di, seed=23)
