@@ -1,5 +1,6 @@
 """Parity of the HIP migration path against the CPU oracle, called through the C ABI.
 Bit-exact: pools are compared as raw 16/32-bit patterns."""
+import functools
 import itertools
 import json
 import os
@@ -400,11 +401,16 @@ def test_calls_from_several_host_threads_on_their_own_streams(kvm):
     kvm.reset()
 
 
-@pytest.mark.parametrize("make", [workloads.config3, workloads.config4])
+@pytest.mark.parametrize("make", [
+    workloads.config3, workloads.config4,
+    functools.partial(workloads.config3, fresh_pools=True), functools.partial(workloads.config4, fresh_pools=True),
+], ids=["cfg3", "cfg4", "cfg3-neighbouring-blocks", "cfg4-neighbouring-blocks"])
 def test_configs_3_and_4_full_size_properties(kvm, make):
     """OPT-13B (TP2 -> TP1) and LLaMA-2-70B GQA (TP2/PP2 -> TP4 rank 1) at full size: after
     every request's call, each of its blocks equals the source rectangles it was sliced from
-    (torch slicing + gather on the GPU); sampled blocks agree with the oracle on the CPU."""
+    (torch slicing + gather on the GPU); sampled blocks agree with the oracle on the CPU.
+    Once with the configurations' scattered block lists and once with the lists of block
+    managers that have just started, whose launches hand out their work in plain order."""
     w = make()
     g = geom_of(w)
     kvm.reset()
