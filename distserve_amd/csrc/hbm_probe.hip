@@ -12,8 +12,11 @@
 // and writes dst + t * tile_bytes, so (run, stride) = (8 KiB, 16 KiB) is the source pattern
 // of a decoding rank that wants two of a context rank's four heads, and run == stride is a
 // dense stream.  There are no index tables, no segments and no division: addresses come
-// from shifts of the workgroup id.  Launches rotate over windows of the buffers so that no
-// launch finds its bytes in the 256 MB last-level cache.
+// from shifts of the workgroup id (sections 1 and 2 of the output; the sources can also be
+// regions scattered over the buffer).  Section 3 adds what sections 1 and 2 leave out of the
+// real copy, block tables and the pools' geometry, in the plainest form: table_kernel below,
+// with the geometry in template constants.  Launches rotate over windows of the buffers, or
+// draw fresh block lists, so that no launch finds its bytes in the 256 MB last-level cache.
 //
 // Build: hipcc --offload-arch=gfx950 -O3 hbm_probe.hip -o hbm_probe (distserve_amd/csrc/build.py does it).
 
