@@ -396,14 +396,26 @@ def main():
     # configuration follows in its own pools and rides along in "configs".
     out, w2 = bench_migrate(2, "request", args.steps, args.warmup, verify_result, args.calibrate_copy)
     configs = {}
+    # every entry below rides along: one that fails says so in its place and costs neither the
+    # headline above nor the entries after it
+    def failed(e):
+        import torch as _torch
+
+        _torch.cuda.empty_cache()
+        return {"error": f"{type(e).__name__}: {e}"}
+
     for cfg, pattern in ((2, "batch"), (1, "request"), (3, "request"), (3, "batch"), (4, "request"), (4, "batch")):
-        d, _ = bench_migrate(cfg, pattern, args.steps, args.warmup, verify_result)
         key = f"cfg{cfg}" if pattern == "request" else f"cfg{cfg}_batched"
-        configs[key] = compact(d)
-    swap = run_swap_bench(args, default_only=True)
-    configs["cfg5"] = swap
-    # configuration 2's shape out of pools that a child process holds; it rides along, and a box
-    # that cannot start the child costs this entry only, not the line
+        try:
+            d, _ = bench_migrate(cfg, pattern, args.steps, args.warmup, verify_result)
+            configs[key] = compact(d)
+        except Exception as e:      # noqa: BLE001
+            configs[key] = failed(e)
+    try:
+        configs["cfg5"] = run_swap_bench(args, default_only=True)
+    except Exception as e:          # noqa: BLE001
+        configs["cfg5"] = failed(e)
+    # configuration 2's shape out of pools that a child process holds
     try:
         ipc = run_ipc_bench(args)
         configs["cfg2_ipc"] = {"GBps": ipc["value"], "frac": ipc["frac_of_hbm_peak"],
@@ -411,8 +423,8 @@ def main():
                                "other_over_this_process": ipc["other_over_this_process"],
                                "us_per_call": ipc["us_per_call"]["other_process"], "bit_exact": ipc["bit_exact"],
                                "pattern": "64-block calls out of 1.75 GiB pools held by a child process (hipIpc mapping)"}
-    except Exception as e:      # noqa: BLE001 - reported, not hidden
-        configs["cfg2_ipc"] = {"error": f"{type(e).__name__}: {e}"}
+    except Exception as e:      # noqa: BLE001
+        configs["cfg2_ipc"] = failed(e)
     # the whole hand-off at configuration 2 (block allocation, the torch op, release of the context
     # blocks), driven by the decoding scheduler, with the transmission time the lifetime events give
     import copy
@@ -426,8 +438,8 @@ def main():
             "transmission_us_per_request_stamped_at_enqueue", "frac_of_hbm_peak", "block_tables_equal_workload",
             "bit_exact")}
         configs["cfg2_handoff"].update(GBps=h["value"], pattern=h["config"]["pattern"])
-    except Exception as e:      # noqa: BLE001 - reported, not hidden: the headline above is already measured
-        configs["cfg2_handoff"] = {"error": f"{type(e).__name__}: {e}"}
+    except Exception as e:      # noqa: BLE001
+        configs["cfg2_handoff"] = failed(e)
     out["configs"] = configs
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(w2)
