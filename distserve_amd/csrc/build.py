@@ -2,7 +2,9 @@
 
 ``libkvmove.so``        hand-written HIP kernels + the C ABI (``include/kvmove.h``); no torch.
 ``libkvmove_torch.so``  torch op shim registering ``block_migration_ops`` / ``swapping_ops``.
-``hbm_probe``           stand-alone program: what plain one-shot kernels reach on the copy's address patterns.
+``tests/lib_explore/libkvmove.so``  the HIP library again with ``-DKVM_EXPLORE``: every kernel flavour and the
+                        knobs that select them, for sweeps and for the tests that show every flavour copies the
+                        same bytes.  Never loaded by the package.
 ``libkvmove_torch_alt.so``  the same ops as ``kvmove_block_migration_ops`` / ``kvmove_swapping_ops``,
                         for a process that keeps another registration of DistServe's names.
 
@@ -26,7 +28,7 @@ INCLUDE_DIR = os.path.join(REPO_DIR, "include")
 KVMOVE_LIB = os.path.join(LIB_DIR, "libkvmove.so")
 TORCH_LIB = os.path.join(LIB_DIR, "libkvmove_torch.so")
 TORCH_ALT_LIB = os.path.join(LIB_DIR, "libkvmove_torch_alt.so")
-HBM_PROBE = os.path.join(LIB_DIR, "hbm_probe")
+EXPLORE_LIB = os.path.join(REPO_DIR, "tests", "lib_explore", "libkvmove.so")
 ALT_NAMESPACES = ("kvmove_block_migration_ops", "kvmove_swapping_ops")
 
 GPU_ARCH = "gfx950"
@@ -44,28 +46,17 @@ def _run(cmd):
         raise RuntimeError(f"build step failed with exit code {res.returncode}: {' '.join(cmd)}")
 
 
-def build_kvmove() -> str:
+def build_kvmove(explore: bool = False) -> str:
     hipcc = shutil.which("hipcc") or os.path.join(ROCM_HOME, "bin", "hipcc")
-    os.makedirs(LIB_DIR, exist_ok=True)
+    out = EXPLORE_LIB if explore else KVMOVE_LIB
+    os.makedirs(os.path.dirname(out), exist_ok=True)
     _run([
         hipcc, f"--offload-arch={GPU_ARCH}", "-O3", "-std=c++17", "-fPIC", "-shared",
         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-        "-Wall", "-Wextra", f"-I{INCLUDE_DIR}",
-        os.path.join(CSRC_DIR, "kvmove.hip"), "-o", KVMOVE_LIB,
+        "-Wall", "-Wextra", f"-I{INCLUDE_DIR}", *(["-DKVM_EXPLORE"] if explore else []),
+        os.path.join(CSRC_DIR, "kvmove.hip"), "-o", out,
     ])
-    return KVMOVE_LIB
-
-
-def build_hbm_probe() -> str:
-    """The stand-alone ceiling probe (``hbm_probe.hip``): a program, not part of the library."""
-    hipcc = shutil.which("hipcc") or os.path.join(ROCM_HOME, "bin", "hipcc")
-    os.makedirs(LIB_DIR, exist_ok=True)
-    _run([
-        hipcc, f"--offload-arch={GPU_ARCH}", "-O3", "-std=c++17",
-        "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wall", "-Wextra",
-        os.path.join(CSRC_DIR, "hbm_probe.hip"), "-o", HBM_PROBE,
-    ])
-    return HBM_PROBE
+    return out
 
 
 def build_torch_shim(alt: bool = False) -> str:
@@ -93,12 +84,12 @@ def build_torch_shim(alt: bool = False) -> str:
 
 def build_all() -> None:
     build_kvmove()
+    build_kvmove(explore=True)
     build_torch_shim()
     build_torch_shim(alt=True)
-    build_hbm_probe()
 
 
 if __name__ == "__main__":
     build_all()
-    print("built:", KVMOVE_LIB, TORCH_LIB, TORCH_ALT_LIB, HBM_PROBE)
+    print("built:", KVMOVE_LIB, TORCH_LIB, TORCH_ALT_LIB, EXPLORE_LIB)
     sys.exit(0)

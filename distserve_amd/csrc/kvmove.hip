@@ -23,17 +23,20 @@
 #include <cstring>
 #include <map>
 #include <mutex>
+#include <shared_mutex>
 #include <string>
 #include <tuple>
 #include <vector>
+#include <time.h>
 #include <unistd.h>
 
 namespace {
 
 // ------------------------------------------------------------------ kernel argument
 
-constexpr int kMaxSegs = 8;    // source segments per launch
-constexpr int kMaxIdx = 432;   // block-index pairs per launch (keeps the argument <= 4 KiB)
+constexpr int kMaxSegs = 8;          // source segments per launch
+constexpr int kMaxIdx = 432;         // block-index pairs per launch as two int32 (keeps the argument <= 4 KiB)
+constexpr int kMaxIdxPacked = 864;   // ... as two uint16 in one word, when both pools have at most 65536 blocks
 
 // One rectangle of the decoding rank's block that a single context rank supplies:
 // n_rows runs of run_bytes, one per overlapping layer.
@@ -77,7 +80,10 @@ struct MigrateArgs {
     uint32_t work;                // W = T * nidx work items per pool kind
     uint32_t work_padded;         // grid.x / 2: W rounded up so that every XCD gets whole chunks
     Seg seg[kMaxSegs];
-    IdxPair idx[kMaxIdx];
+    union {
+        IdxPair idx[kMaxIdx];
+        uint32_t packed[kMaxIdxPacked];   // context block | decoding block << 16
+    };
 };
 static_assert(sizeof(MigrateArgs) <= 4096, "kernel argument must stay within 4 KiB");
 
@@ -214,12 +220,27 @@ __device__ __forceinline__ uint32_t fast_div(uint32_t n, uint32_t magic, uint32_
     return (t + ((n - t) >> (shifts & 0xffu))) >> (shifts >> 8);
 }
 
+// The index pair of one block, from either form of the table.
+template <bool PACKED>
+__device__ __forceinline__ void load_pair(const MigrateArgs &a, uint32_t pair, uint32_t &ctx, uint32_t &dec)
+{
+    if constexpr (PACKED) {
+        const uint32_t p = a.packed[pair];
+        ctx = p & 0xffffu;
+        dec = p >> 16;
+    } else {
+        const IdxPair ix = a.idx[pair];
+        ctx = (uint32_t)ix.ctx;
+        dec = (uint32_t)ix.dec;
+    }
+}
+
 // One tile of one block of one pool kind.  Everything up to the lane offset is
 // wave-uniform and lives in SGPRs.  The scalar loads are arranged for a short dependent
 // chain, because a workgroup here lives for little more than one memory round trip: the
 // header (with every segment's tile range) and the block-index pair are independent
 // loads, the segment's fields are the one dependent round after them.
-template <typename V, int THREADS, int UNROLL, int FLAGS>
+template <typename V, int THREADS, int UNROLL, int FLAGS, bool PACKED>
 __device__ __forceinline__ void do_tile(const MigrateArgs &a, const u32x16 h, uint32_t tile, uint32_t pair, bool is_v)
 {
     // `h` is the first header record (64 bytes, one 16-dword scalar load by the caller); the
@@ -227,7 +248,8 @@ __device__ __forceinline__ void do_tile(const MigrateArgs &a, const u32x16 h, ui
     // {header records} -> {index pair, segment} -> addresses.
     static_assert(offsetof(MigrateArgs, tile_end) == 32 && offsetof(MigrateArgs, tiles_per_block) == 64 &&
                       offsetof(MigrateArgs, seg) == 96, "header layout");
-    const IdxPair ix = a.idx[pair];
+    uint32_t ctx, dec;
+    load_pair<PACKED>(a, pair, ctx, dec);
     uint32_t s = 0, tile_begin = 0;
 #pragma unroll
     for (int j = 0; j < kMaxSegs - 1; ++j) {
@@ -244,8 +266,8 @@ __device__ __forceinline__ void do_tile(const MigrateArgs &a, const u32x16 h, ui
     const uint32_t src_row_stride = g[6], dst_row_stride = g[7], dst_off = g[8], run_bytes = g[9];
     const uint32_t n_rows = g[10], rows_per_tile = g[11], pieces_per_row = g[12], piece_bytes = g[13];
 
-    const gchar *src = reinterpret_cast<const gchar *>(src_base + (uint64_t)(uint32_t)ix.ctx * src_block_stride);
-    gchar *dst = reinterpret_cast<gchar *>(dst_base + (uint64_t)(uint32_t)ix.dec * dst_block_stride + dst_off);
+    const gchar *src = reinterpret_cast<const gchar *>(src_base + (uint64_t)ctx * src_block_stride);
+    gchar *dst = reinterpret_cast<gchar *>(dst_base + (uint64_t)dec * dst_block_stride + dst_off);
 
     if (rows_per_tile == 1) {
         const uint32_t row = fast_div(tile, g[14], g[15]);
@@ -271,7 +293,7 @@ __device__ __forceinline__ void do_tile(const MigrateArgs &a, const u32x16 h, ui
 // into a work item such that each XCD walks its own contiguous chunks of `chunk_tiles`
 // tiles (chunk number seq / C * 8 + xcd).  Chunks of 256 KiB and more measured 2-3 % faster
 // than in-order ids, chunks of 2-64 KiB 5-10 % slower.
-template <typename V, int THREADS, int UNROLL, int FLAGS>
+template <typename V, int THREADS, int UNROLL, int FLAGS, bool PACKED>
 __global__ __launch_bounds__(THREADS) void kvm_copy_kernel(const MigrateArgs a)
 {
     // both header records in one round of scalar loads
@@ -292,14 +314,14 @@ __global__ __launch_bounds__(THREADS) void kvm_copy_kernel(const MigrateArgs a)
     // behind the branch.
     if (w >= work || h[7] == 0) return;
     const uint32_t pair = fast_div(w, m[1], m[2]);
-    do_tile<V, THREADS, UNROLL, FLAGS>(a, h, w - pair * tiles_per_block, pair, is_v);
+    do_tile<V, THREADS, UNROLL, FLAGS, PACKED>(a, h, w - pair * tiles_per_block, pair, is_v);
 }
 
 // The same for the plainest shape: one segment whose rows collapsed into a single run that
 // is a whole number of full tiles (context and decoding layouts agree, e.g. TP1 -> TP1).
 // Nothing depends on the tile's position but two multiplications, so the scalar prologue is
 // one round of loads for the three records, the index pair, and a dozen SALU instructions.
-template <typename V, int THREADS, int UNROLL, int FLAGS>
+template <typename V, int THREADS, int UNROLL, int FLAGS, bool PACKED>
 __global__ __launch_bounds__(THREADS) void kvm_copy_simple_kernel(const MigrateArgs a)
 {
     constexpr uint32_t kTile = THREADS * UNROLL * (uint32_t)sizeof(V);
@@ -319,12 +341,13 @@ __global__ __launch_bounds__(THREADS) void kvm_copy_simple_kernel(const MigrateA
     if (w >= work || h[7] == 0 || g[10] == 0) return;   // (names h and g: see kvm_copy_kernel)
     const uint32_t pair = fast_div(w, m[1], m[2]);
     const uint32_t tile = w - pair * tiles_per_block;
-    const IdxPair ix = a.idx[pair];
+    uint32_t ctx, dec;
+    load_pair<PACKED>(a, pair, ctx, dec);
     const uint64_t src_base = is_v ? u64_of(g[2], g[3]) : u64_of(g[0], g[1]);
     const uint64_t dst_base = is_v ? u64_of(h[2], h[3]) : u64_of(h[0], h[1]);
     const uint64_t off = (uint64_t)tile * kTile;
-    const gchar *src = reinterpret_cast<const gchar *>(src_base + (uint64_t)(uint32_t)ix.ctx * u64_of(g[4], g[5]) + off);
-    gchar *dst = reinterpret_cast<gchar *>(dst_base + (uint64_t)(uint32_t)ix.dec * u64_of(h[4], h[5]) + g[8] + off);
+    const gchar *src = reinterpret_cast<const gchar *>(src_base + (uint64_t)ctx * u64_of(g[4], g[5]) + off);
+    gchar *dst = reinterpret_cast<gchar *>(dst_base + (uint64_t)dec * u64_of(h[4], h[5]) + g[8] + off);
     V r[UNROLL];
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u)
@@ -338,14 +361,14 @@ __global__ __launch_bounds__(THREADS) void kvm_copy_simple_kernel(const MigrateA
 // (block, tile) pairs of the launch with a stride of gridDim.x.  A copy that the host link
 // limits to tens of GB/s needs only a handful of workgroups in flight, and leaves the rest
 // of the GPU to whatever runs beside it.
-template <typename V>
-__global__ __launch_bounds__(256) void kvm_walk_kernel(const MigrateArgs a, uint32_t tiles_per_block)
+template <typename V, bool PACKED, int THREADS, int UNROLL>
+__global__ __launch_bounds__(THREADS) void kvm_walk_kernel(const MigrateArgs a, uint32_t tiles_per_block)
 {
     const uint32_t total = a.nidx * tiles_per_block;
     for (uint32_t w = blockIdx.x; w < total; w += gridDim.x) {
         const uint32_t pair = w / tiles_per_block;
-        do_tile<V, 256, 4, kNtLoad | kNtStore>(a, *reinterpret_cast<const u32x16 *>(&a), w - pair * tiles_per_block,
-                                               pair, blockIdx.y != 0);
+        do_tile<V, THREADS, UNROLL, kNtLoad | kNtStore, PACKED>(a, *reinterpret_cast<const u32x16 *>(&a),
+                                                                w - pair * tiles_per_block, pair, blockIdx.y != 0);
     }
 }
 
@@ -372,37 +395,67 @@ int fail(int code, const char *fmt, ...)
     } while (0)
 
 // ---- options
+//
+// The library ships one flavour of the copy kernel (a single-wave workgroup that moves 1 KiB,
+// nontemporal both ways: the one every sweep chose) and the options a deployment may want to
+// set.  The exploration build (-DKVM_EXPLORE, used by sweeps and by the tests that show every
+// flavour copies the same bytes) adds the other flavours and the knobs that select them.
 
+std::atomic<int64_t> opt_swap_mode{3};
+std::atomic<int64_t> opt_swap_wgs{16};
+std::atomic<int64_t> opt_swap_wgs_in{16};
+std::atomic<int64_t> opt_swap_kernel_below{1ll << 32};
+std::atomic<int64_t> opt_xcd_map{1};
+std::atomic<int64_t> opt_sort_pairs{1};
+#ifdef KVM_EXPLORE
 std::atomic<int64_t> opt_tile_bytes{0};
 std::atomic<int64_t> opt_threads{64};
 std::atomic<int64_t> opt_unroll{1};
 std::atomic<int64_t> opt_nt_load{1};
 std::atomic<int64_t> opt_nt_store{1};
-std::atomic<int64_t> opt_swap_mode{3};
-std::atomic<int64_t> opt_swap_wgs{8};
-std::atomic<int64_t> opt_swap_wgs_in{10};
-std::atomic<int64_t> opt_swap_kernel_below{1ll << 32};
 std::atomic<int64_t> opt_lds_pad{0};
 std::atomic<int64_t> opt_wave_contig{0};
-std::atomic<int64_t> opt_xcd_map{1};
 std::atomic<int64_t> opt_simple{1};
+std::atomic<int64_t> opt_max_pairs{kMaxIdxPacked};
+std::atomic<int64_t> opt_packed{1};
+std::atomic<int64_t> opt_swap_threads{256};
+std::atomic<int64_t> opt_swap_unroll{1};
+int64_t tune_tile_bytes() { return opt_tile_bytes.load(); }
+int64_t tune_lds_pad() { return opt_lds_pad.load(); }
+bool tune_simple() { return opt_simple.load() != 0; }
+int64_t tune_max_pairs() { return opt_max_pairs.load(); }
+bool tune_packed() { return opt_packed.load() != 0; }
+#else
+constexpr int64_t tune_tile_bytes() { return 0; }
+constexpr int64_t tune_lds_pad() { return 0; }
+constexpr bool tune_simple() { return true; }
+constexpr int64_t tune_max_pairs() { return kMaxIdxPacked; }
+constexpr bool tune_packed() { return true; }
+#endif
 
 std::atomic<int64_t> *find_opt(const char *name)
 {
     if (!name) return nullptr;
+    if (!strcmp(name, "swap_mode")) return &opt_swap_mode;
+    if (!strcmp(name, "swap_wgs")) return &opt_swap_wgs;
+    if (!strcmp(name, "swap_wgs_in")) return &opt_swap_wgs_in;
+    if (!strcmp(name, "swap_kernel_below")) return &opt_swap_kernel_below;
+    if (!strcmp(name, "xcd_map")) return &opt_xcd_map;
+    if (!strcmp(name, "sort_pairs")) return &opt_sort_pairs;
+#ifdef KVM_EXPLORE
     if (!strcmp(name, "tile_bytes")) return &opt_tile_bytes;
     if (!strcmp(name, "threads")) return &opt_threads;
     if (!strcmp(name, "unroll")) return &opt_unroll;
     if (!strcmp(name, "nt_load")) return &opt_nt_load;
     if (!strcmp(name, "nt_store")) return &opt_nt_store;
-    if (!strcmp(name, "swap_mode")) return &opt_swap_mode;
-    if (!strcmp(name, "swap_wgs")) return &opt_swap_wgs;
-    if (!strcmp(name, "swap_wgs_in")) return &opt_swap_wgs_in;
-    if (!strcmp(name, "swap_kernel_below")) return &opt_swap_kernel_below;
     if (!strcmp(name, "lds_pad")) return &opt_lds_pad;
     if (!strcmp(name, "wave_contig")) return &opt_wave_contig;
-    if (!strcmp(name, "xcd_map")) return &opt_xcd_map;
     if (!strcmp(name, "simple")) return &opt_simple;
+    if (!strcmp(name, "max_pairs")) return &opt_max_pairs;
+    if (!strcmp(name, "packed")) return &opt_packed;
+    if (!strcmp(name, "swap_threads")) return &opt_swap_threads;
+    if (!strcmp(name, "swap_unroll")) return &opt_swap_unroll;
+#endif
     return nullptr;
 }
 
@@ -418,27 +471,37 @@ struct Source {
 
 using SourceKey = std::tuple<int64_t, int32_t, int32_t>;
 
-std::mutex g_mu;
+// g_mu guards g_sources.  A migrate call holds it shared from the lookup of its pools until its
+// last launch is enqueued, so that a mapping it reads through cannot be closed in between;
+// registrations and resets take it exclusively, and only for the insert of a binding or for
+// the sequence {drop bindings, wait for the device, unmap}.  g_reg_mu serialises registrations
+// and resets among themselves (they may map memory and wait for the device, with g_mu free);
+// g_opened is only touched under it.
+std::shared_mutex g_mu;
+std::mutex g_reg_mu;
 std::map<SourceKey, Source> g_sources;
 
 // Allocations of other processes that registration has mapped into this one.  One entry per
 // (exporting process, allocation): hipIpcOpenMemHandle is called once however many pools lie
-// in the allocation, and the mapping stays until kvm_reset.
+// in the allocation, and the mapping stays while a registered pool lies in it.
 struct Opened {
-    int64_t pid, remote_base, size;
-    int64_t serial;   // the exporter's id of the allocation; a new allocation at an old address has another
+    int64_t pid, nonce, remote_base, size;
+    int64_t serial;      // the exporter's id of the allocation (0 = it had none to give)
+    uint64_t opened_in;  // the registration call that opened it
     char *local_base;
 };
-std::vector<Opened> g_opened;   // guarded by g_mu
+std::vector<Opened> g_opened;
+uint64_t g_reg_call = 0;        // counts registration calls; guarded by g_reg_mu
 
 // Handle words (int64 each).
 enum {
     kHwMagic = 0, kHwPid, kHwDevice, kHwPtr, kHwBytes, kHwAllocBase, kHwAllocSize, kHwFlags,
     kHwIpc = 8,                                  // 8 words = the 64 bytes of a hipIpcMemHandle_t
-    kHwCheck = 16,
+    kHwNonce = 16,
+    kHwCheck = 17,
 };
 static_assert(sizeof(hipIpcMemHandle_t) == 64 && kHwCheck + 1 == KVM_HANDLE_WORDS, "handle layout");
-constexpr int64_t kHandleMagic = 0x4b564d4f56453033LL;  // "KVMOVE03"
+constexpr int64_t kHandleMagic = 0x4b564d4f56453034LL;  // "KVMOVE04"
 constexpr int64_t kHandleHasIpc = 1;                    // flag: words 8..15 hold an exported IPC handle
 // The flags word carries the flags in its low byte and, above it, the runtime's id of the
 // allocation in the exporting process (HIP_POINTER_ATTRIBUTE_BUFFER_ID: every allocation of
@@ -454,37 +517,57 @@ int64_t handle_check(const int64_t *h)
     return (int64_t)x;
 }
 
+// A random word drawn once per process.  A handle is "this process's own", and resolves to
+// its pointer without any mapping, only when pid AND nonce match: two processes in different
+// pid namespaces (two containers that are both pid 1) share a pid but not a nonce.
+int64_t process_nonce()
+{
+    static const int64_t nonce = [] {
+        uint64_t x = 0;
+        if (FILE *f = fopen("/dev/urandom", "rb")) {
+            if (fread(&x, sizeof x, 1, f) != 1) x = 0;
+            fclose(f);
+        }
+        timespec ts{};
+        clock_gettime(CLOCK_MONOTONIC, &ts);
+        x ^= ((uint64_t)getpid() << 32) ^ (uint64_t)ts.tv_nsec ^ ((uint64_t)ts.tv_sec << 20) ^ (uint64_t)(uintptr_t)&x;
+        return (int64_t)(x | 1);
+    }();
+    return nonce;
+}
+
+bool is_own_handle(const int64_t *h) { return h[kHwPid] == (int64_t)getpid() && h[kHwNonce] == process_nonce(); }
+
 // ---- kernel table
 
 using KernelFn = void (*)(const MigrateArgs);
 
 struct Variant {
     int threads, unroll, flags;
-    KernelFn fn;         // any shape
-    KernelFn simple_fn;  // one collapsed segment of full tiles
+    KernelFn fn[2];         // any shape; [1] reads the packed index table
+    KernelFn simple_fn[2];  // one collapsed segment of full tiles
 };
 
-#define KVM_VARIANT(T, U, F) {T, U, F, kvm_copy_kernel<u32x4, T, U, F>, kvm_copy_simple_kernel<u32x4, T, U, F>}
+#define KVM_VARIANT(T, U, F)                                                                     \
+    {T, U, F, {kvm_copy_kernel<u32x4, T, U, F, false>, kvm_copy_kernel<u32x4, T, U, F, true>},      \
+     {kvm_copy_simple_kernel<u32x4, T, U, F, false>, kvm_copy_simple_kernel<u32x4, T, U, F, true>}}
 #define KVM_VARIANT_ROW(T, F) \
     KVM_VARIANT(T, 1, F), KVM_VARIANT(T, 2, F), KVM_VARIANT(T, 4, F), KVM_VARIANT(T, 8, F), KVM_VARIANT(T, 16, F)
 
-// 16-byte-vector flavours that are compiled in.  The exploration build (-DKVM_EXPLORE)
-// carries the whole grid for sweeps; the shipped library carries the one the sweeps chose
-// (64 lanes, one vector per lane: a single-wave workgroup that moves 1 KiB) plus a few
-// neighbours so that the tuning tests can show every flavour copies the same bytes.
+// 16-byte-vector flavours that are compiled in: the one the sweeps chose (64 lanes, one
+// vector per lane: a single-wave workgroup that moves 1 KiB), and in the exploration build
+// the grid the sweeps ran over.
 const Variant kVariants[] = {
+    KVM_VARIANT(64, 1, 3),
 #ifdef KVM_EXPLORE
-    KVM_VARIANT_ROW(64, 3),   KVM_VARIANT_ROW(128, 3),  KVM_VARIANT_ROW(256, 3),
-    KVM_VARIANT_ROW(512, 3),  KVM_VARIANT_ROW(1024, 3),
+    KVM_VARIANT(64, 2, 3),    KVM_VARIANT(64, 4, 3),    KVM_VARIANT(64, 8, 3),   KVM_VARIANT(64, 16, 3),
+    KVM_VARIANT_ROW(128, 3),  KVM_VARIANT_ROW(256, 3),  KVM_VARIANT_ROW(512, 3), KVM_VARIANT_ROW(1024, 3),
     KVM_VARIANT_ROW(64, 7),   KVM_VARIANT_ROW(128, 7),  KVM_VARIANT_ROW(256, 7),
     KVM_VARIANT_ROW(512, 7),  KVM_VARIANT_ROW(1024, 7),
+    KVM_VARIANT(64, 1, 0),    KVM_VARIANT(64, 1, 1),    KVM_VARIANT(64, 1, 2),
     KVM_VARIANT(256, 4, 0),   KVM_VARIANT(256, 4, 1),   KVM_VARIANT(256, 4, 2),
     KVM_VARIANT(256, 8, 0),   KVM_VARIANT(256, 8, 1),   KVM_VARIANT(256, 8, 2),
-#else
-    KVM_VARIANT(64, 1, 3),   KVM_VARIANT(64, 2, 3),   KVM_VARIANT(128, 1, 3),  KVM_VARIANT(256, 1, 3),
-    KVM_VARIANT(256, 4, 3),  KVM_VARIANT(256, 8, 3),  KVM_VARIANT(512, 2, 3),  KVM_VARIANT(512, 8, 3),
-    KVM_VARIANT(1024, 4, 3), KVM_VARIANT(64, 1, 0),   KVM_VARIANT(256, 4, 0),  KVM_VARIANT(512, 8, 0),
-    KVM_VARIANT(64, 4, 7),   KVM_VARIANT(256, 8, 7),
+    KVM_VARIANT(512, 8, 0),
 #endif
 };
 
@@ -496,28 +579,32 @@ struct Launch {
     int vec = 0;
 };
 
-int pick_kernel(int vec, Launch *l)
+int pick_kernel(int vec, bool packed, Launch *l)
 {
     l->vec = vec;
     if (vec != 16) {
         // narrow vectors only serve odd shapes and misaligned pools: one flavour each
         l->threads = 256;
         l->unroll = 4;
-        l->fn = vec == 8 ? kvm_copy_kernel<u32x2, 256, 4, 3>
-              : vec == 4 ? kvm_copy_kernel<uint32_t, 256, 4, 3>
-              : vec == 2 ? kvm_copy_kernel<uint16_t, 256, 4, 3>
-                         : kvm_copy_kernel<uint8_t, 256, 4, 3>;
+        l->fn = vec == 8 ? (packed ? kvm_copy_kernel<u32x2, 256, 4, 3, true> : kvm_copy_kernel<u32x2, 256, 4, 3, false>)
+              : vec == 4 ? (packed ? kvm_copy_kernel<uint32_t, 256, 4, 3, true> : kvm_copy_kernel<uint32_t, 256, 4, 3, false>)
+              : vec == 2 ? (packed ? kvm_copy_kernel<uint16_t, 256, 4, 3, true> : kvm_copy_kernel<uint16_t, 256, 4, 3, false>)
+                         : (packed ? kvm_copy_kernel<uint8_t, 256, 4, 3, true> : kvm_copy_kernel<uint8_t, 256, 4, 3, false>);
         return KVM_OK;
     }
+#ifdef KVM_EXPLORE
     const int threads = (int)opt_threads.load(), unroll = (int)opt_unroll.load();
     const int flags = (opt_nt_load.load() ? kNtLoad : 0) | (opt_nt_store.load() ? kNtStore : 0) |
                       (opt_wave_contig.load() ? kWaveContig : 0);
+#else
+    const int threads = 64, unroll = 1, flags = kNtLoad | kNtStore;
+#endif
     for (const Variant &v : kVariants) {
         if (v.threads == threads && v.unroll == unroll && v.flags == flags) {
             l->threads = threads;
             l->unroll = unroll;
-            l->fn = v.fn;
-            l->simple_fn = v.simple_fn;
+            l->fn = v.fn[packed];
+            l->simple_fn = v.simple_fn[packed];
             return KVM_OK;
         }
     }
@@ -605,6 +692,7 @@ int check_geom(const KvmGeom *g)
 
 // `arithmetic_only`: context ranks that are not registered count as 16-byte aligned pools of
 // unknown size at address 0, so that the launch shape can be computed without a device.
+// The caller holds g_mu (shared) and keeps it until the plan's pointers are no longer used.
 int build_plan(const KvmGeom *g, const void *dst_k, const void *dst_v, Plan *plan, bool arithmetic_only = false)
 {
     if (int rc = check_geom(g)) return rc;
@@ -624,7 +712,6 @@ int build_plan(const KvmGeom *g, const void *dst_k, const void *dst_v, Plan *pla
     plan->min_src_blocks = INT64_MAX;
     uint64_t align_bits = (uint64_t)head_bytes | (uint64_t)(uintptr_t)dst_k | (uint64_t)(uintptr_t)dst_v;
 
-    std::lock_guard<std::mutex> lock(g_mu);
     for (int64_t p = l0 / Lc; p * Lc < l1; ++p) {
         for (int64_t t = h0 / Hc; t * Hc < h1; ++t) {
             auto it = g_sources.find(SourceKey{g->ctx_instance, (int32_t)p, (int32_t)t});
@@ -700,13 +787,44 @@ void plan_work(MigrateArgs &args, uint32_t tiles, uint32_t tile_bytes, bool neig
 
 using WalkFn = void (*)(const MigrateArgs, uint32_t);
 
-WalkFn pick_walk(int vec)
+// The link-bound form's workgroup: 256 lanes that move one 16-byte vector each per step
+// (4 KiB per workgroup in flight; narrower vectors move four per lane to keep about as many
+// bytes in flight).  Many light workgroups fill the link as well as few heavy ones with the
+// same bytes in flight, and disturb HBM-bound kernels beside them less: measured at the
+// LLaMA-2-7B slab size, 16 workgroups of 4 KiB against 8 to 10 of 16 KiB: the same 99 % of the
+// link alone, a migration beside a swap-in 2.4 % slower instead of 8.6 %, and 46 GB/s each
+// way instead of 34 / 49 when a swap-out and a swap-in are in flight together.
+WalkFn pick_walk(int vec, bool packed, int *threads, int *unroll)
 {
-    return vec == 16 ? kvm_walk_kernel<u32x4>
-         : vec == 8  ? kvm_walk_kernel<u32x2>
-         : vec == 4  ? kvm_walk_kernel<uint32_t>
-         : vec == 2  ? kvm_walk_kernel<uint16_t>
-                     : kvm_walk_kernel<uint8_t>;
+    *threads = 256;
+    *unroll = vec == 16 ? 1 : 4;
+#ifdef KVM_EXPLORE
+    // other workgroup shapes, 16-byte vectors and packed tables only
+    if (vec == 16 && packed) {
+        const int64_t t = opt_swap_threads.load(), u = opt_swap_unroll.load();
+        WalkFn fn = nullptr;
+#define KVM_WALK(T, U) if (t == T && u == U) fn = kvm_walk_kernel<u32x4, true, T, U>;
+        KVM_WALK(64, 1) KVM_WALK(64, 2) KVM_WALK(64, 4) KVM_WALK(128, 1) KVM_WALK(128, 2) KVM_WALK(128, 4)
+        KVM_WALK(256, 2) KVM_WALK(256, 4) KVM_WALK(256, 8) KVM_WALK(512, 4) KVM_WALK(1024, 4)
+#undef KVM_WALK
+        if (fn) {
+            *threads = (int)t;
+            *unroll = (int)u;
+            return fn;
+        }
+    }
+#endif
+    if (packed)
+        return vec == 16 ? kvm_walk_kernel<u32x4, true, 256, 1>
+             : vec == 8  ? kvm_walk_kernel<u32x2, true, 256, 4>
+             : vec == 4  ? kvm_walk_kernel<uint32_t, true, 256, 4>
+             : vec == 2  ? kvm_walk_kernel<uint16_t, true, 256, 4>
+                         : kvm_walk_kernel<uint8_t, true, 256, 4>;
+    return vec == 16 ? kvm_walk_kernel<u32x4, false, 256, 1>
+         : vec == 8  ? kvm_walk_kernel<u32x2, false, 256, 4>
+         : vec == 4  ? kvm_walk_kernel<uint32_t, false, 256, 4>
+         : vec == 2  ? kvm_walk_kernel<uint16_t, false, 256, 4>
+                     : kvm_walk_kernel<uint8_t, false, 256, 4>;
 }
 
 // Everything launch_copy decides about one group of up to 8 segments before it launches.
@@ -720,29 +838,46 @@ struct Group {
 // A launch is a 1-D grid of 2 * work_padded workgroups of `threads` lanes, and the runtime
 // refuses a grid of 2^32 work-items or more.  plan_work pads the work of a launch by fewer
 // than 8 tiles, or not at all, so this many index pairs per launch stay below that.
-int64_t pairs_per_launch(uint32_t tiles, int threads)
+int64_t pairs_per_launch(uint32_t tiles, int threads, bool packed)
 {
     const int64_t max_tiles = (int64_t)(UINT32_MAX / (2u * (uint32_t)threads)) - 8;
-    return std::min<int64_t>(kMaxIdx, max_tiles / (int64_t)tiles);
+    const int64_t table = std::min<int64_t>(packed ? kMaxIdxPacked : kMaxIdx, tune_max_pairs());
+    return std::min<int64_t>(table, max_tiles / (int64_t)tiles);
 }
 
+// What launch_copy reports about the launches of a call.
+struct CopyShape {
+    int64_t launches = 0;
+    int64_t wgs_per_block = 0;     // workgroups per block, K and V together
+    int64_t max_items = 0;         // work-items of the largest launch
+    int64_t pairs_per_launch = 0;  // index pairs the largest launch carries at most
+    int threads = 0, unroll = 0;
+    bool simple = false;           // the short-prologue kernel serves every launch
+};
+
 // Enqueues the copy over `segs` x `pairs`, as many launches as the 4 KiB argument needs
-// (8 segments and 432 index pairs each) and the grid limit allows.  Every launch of the call
-// is sized and checked before the first one is enqueued, so a call that cannot be launched
-// has touched nothing.  `pairs == nullptr` only counts what would be launched.  walk_wgs > 0
-// selects the link-bound form with that many workgroups per pool kind.
-int launch_copy(std::vector<Seg> segs, const IdxPair *pairs, int64_t n, char *dst_k, char *dst_v,
-                uint64_t dst_block_stride, int vec, hipStream_t stream, int64_t *out_launches,
-                int64_t *out_wgs_per_block, int *out_threads, int walk_wgs = 0, bool *out_simple = nullptr,
-                int64_t *out_max_items = nullptr, bool neighbours = false)
+// (8 segments and 864 packed or 432 wide index pairs each) and the grid limit allows.  Every
+// launch of the call is sized and checked before the first one is enqueued, so a call that
+// cannot be launched has touched nothing.  `pairs == nullptr` only counts what would be
+// launched.  `packed`: every index is below 65536.  walk_wgs > 0 selects the link-bound form
+// with that many workgroups per pool kind.
+int launch_copy(std::vector<Seg> segs, const IdxPair *pairs, int64_t n, bool packed, char *dst_k, char *dst_v,
+                uint64_t dst_block_stride, int vec, hipStream_t stream, CopyShape *shape = nullptr,
+                int walk_wgs = 0, bool neighbours = false)
 {
+    packed = packed && tune_packed();
     Launch k;
-    if (int rc = pick_kernel(vec, &k)) return rc;
+    if (int rc = pick_kernel(vec, packed, &k)) return rc;
     // tile_bytes 0 = one shot: exactly what the workgroup's lanes hold in flight
-    uint32_t tile_bytes = (uint32_t)opt_tile_bytes.load();
-    if (tile_bytes == 0) tile_bytes = (uint32_t)((walk_wgs > 0 ? 256 * 4 : k.threads * k.unroll) * vec);
-    int64_t launches = 0, wgs_per_block = 0, max_items = 0;
-    bool all_simple = true;
+    uint32_t tile_bytes = (uint32_t)tune_tile_bytes();
+    WalkFn walk_fn = nullptr;
+    int walk_threads = 256, walk_unroll = 4;
+    if (walk_wgs > 0) walk_fn = pick_walk(vec, packed, &walk_threads, &walk_unroll);
+    if (tile_bytes == 0) tile_bytes = (uint32_t)((walk_wgs > 0 ? walk_threads * walk_unroll : k.threads * k.unroll) * vec);
+    CopyShape out;
+    out.threads = k.threads;
+    out.unroll = k.unroll;
+    out.simple = !segs.empty();
     std::vector<Group> groups((segs.size() + kMaxSegs - 1) / kMaxSegs);
     for (size_t gi = 0; gi < groups.size(); ++gi) {
         const size_t s0 = gi * kMaxSegs;
@@ -765,74 +900,103 @@ int launch_copy(std::vector<Seg> segs, const IdxPair *pairs, int64_t n, char *ds
         args.tile_end[args.nseg - 1] = UINT32_MAX;   // nothing lies past the last segment
         // one collapsed segment of full one-shot tiles takes the short-prologue kernel
         const Seg &first = args.seg[0];
-        grp.simple = walk_wgs == 0 && k.simple_fn && opt_simple.load() && args.nseg == 1 &&
+        grp.simple = walk_wgs == 0 && k.simple_fn && tune_simple() && args.nseg == 1 &&
                      first.n_rows == 1 && first.rows_per_tile == 1 && first.run_bytes % tile_bytes == 0 &&
                      tile_bytes == (uint32_t)(k.threads * k.unroll * vec);
-        all_simple = all_simple && grp.simple;
-        wgs_per_block += 2 * (int64_t)tiles_total;
+        out.simple = out.simple && grp.simple;
+        out.wgs_per_block += 2 * (int64_t)tiles_total;
         if (tiles_total == 0 || tiles_total > (1u << 29))
             return fail(KVM_EINVAL, "%llu tiles per block cannot be launched", (unsigned long long)tiles_total);
         grp.tiles = (uint32_t)tiles_total;
         // the walking form's grid is a few workgroups whatever the work
-        grp.per_launch = walk_wgs > 0 ? std::min<int64_t>(kMaxIdx, (int64_t)(UINT32_MAX / grp.tiles))
-                                      : pairs_per_launch(grp.tiles, k.threads);
+        grp.per_launch = walk_wgs > 0
+                             ? std::min<int64_t>(packed ? kMaxIdxPacked : kMaxIdx, (int64_t)(UINT32_MAX / grp.tiles))
+                             : pairs_per_launch(grp.tiles, k.threads, packed);
         if (grp.per_launch < 1)
             return fail(KVM_EINVAL, "one block is %u tiles of %d lanes per pool kind: no launch can hold it",
                         grp.tiles, k.threads);
+        out.pairs_per_launch = std::max(out.pairs_per_launch, grp.per_launch);
         const int64_t largest = std::min<int64_t>(grp.per_launch, std::max<int64_t>(n, 1));
         if (walk_wgs > 0) {
-            max_items = std::max<int64_t>(max_items, 2 * 256 * (int64_t)walk_wgs);
+            out.max_items = std::max<int64_t>(out.max_items, 2 * walk_threads * (int64_t)walk_wgs);
         } else {
             args.nidx = (uint32_t)largest;      // the launch loop below sets it again, launch by launch
             plan_work(args, grp.tiles, tile_bytes, neighbours);
             const int64_t items = 2 * (int64_t)args.work_padded * k.threads;
             if (items > (int64_t)UINT32_MAX)
                 return fail(KVM_EINVAL, "a launch of %lld work-items cannot be made", (long long)items);
-            max_items = std::max(max_items, items);
+            out.max_items = std::max(out.max_items, items);
         }
-        launches += n == 0 ? 1 : (n + grp.per_launch - 1) / grp.per_launch;
+        out.launches += n == 0 ? 1 : (n + grp.per_launch - 1) / grp.per_launch;
     }
     if (pairs) {
         for (Group &grp : groups) {
             MigrateArgs &args = grp.args;
             for (int64_t i0 = 0; i0 < n; i0 += grp.per_launch) {
                 args.nidx = (uint32_t)std::min<int64_t>(grp.per_launch, n - i0);
-                memcpy(args.idx, pairs + i0, args.nidx * sizeof(IdxPair));
+                if (packed) {
+                    for (uint32_t i = 0; i < args.nidx; ++i)
+                        args.packed[i] = (uint32_t)pairs[i0 + i].ctx | ((uint32_t)pairs[i0 + i].dec << 16);
+                } else {
+                    memcpy(args.idx, pairs + i0, args.nidx * sizeof(IdxPair));
+                }
                 if (walk_wgs > 0) {
                     const uint32_t work = grp.tiles * args.nidx;
-                    hipLaunchKernelGGL(pick_walk(vec), dim3(std::min<uint32_t>((uint32_t)walk_wgs, work), 2),
-                                       dim3(256), 0, stream, args, grp.tiles);
+                    hipLaunchKernelGGL(walk_fn, dim3(std::min<uint32_t>((uint32_t)walk_wgs, work), 2),
+                                       dim3(walk_threads), 0, stream, args, grp.tiles);
                 } else {
                     plan_work(args, grp.tiles, tile_bytes, neighbours);
                     hipLaunchKernelGGL(grp.simple ? k.simple_fn : k.fn, dim3(2 * args.work_padded), dim3(k.threads),
-                                       (size_t)opt_lds_pad.load(), stream, args);
+                                       (size_t)tune_lds_pad(), stream, args);
                 }
                 KVM_HIP(hipGetLastError());
             }
         }
     }
-    if (out_launches) *out_launches = launches;
-    if (out_wgs_per_block) *out_wgs_per_block = wgs_per_block;
-    if (out_threads) *out_threads = k.threads;
-    if (out_simple) *out_simple = all_simple && !segs.empty();
-    if (out_max_items) *out_max_items = max_items;
+    if (shape) *shape = out;
     return KVM_OK;
 }
 
 // dec index list must not repeat: the copies of one call run concurrently.
 thread_local std::vector<uint64_t> g_seen;
 
-// `neighbours` (optional): whether at least half of the source blocks follow their
-// predecessor in the list directly, i.e. the list is mostly runs of adjacent blocks.
+// Orders the pairs of a call by source block; pairs with the same source keep their order.
+// The copy does not depend on the order of its pairs, the memory system does: a call that
+// names a large part of the source pool reads it front to back instead of at random.
+thread_local std::vector<uint32_t> g_count;
+thread_local std::vector<IdxPair> g_sorted;
+
+void sort_by_source(std::vector<IdxPair> *pairs, int64_t n_src)
+{
+    const size_t n = pairs->size();
+    if ((uint64_t)n_src > 8 * (uint64_t)n + 1024) {
+        std::stable_sort(pairs->begin(), pairs->end(), [](const IdxPair &x, const IdxPair &y) { return x.ctx < y.ctx; });
+        return;
+    }
+    // counting sort: O(n + n_src)
+    g_count.assign((size_t)n_src + 1, 0);
+    for (const IdxPair &p : *pairs) ++g_count[(size_t)p.ctx + 1];
+    for (size_t b = 0; b < (size_t)n_src; ++b) g_count[b + 1] += g_count[b];
+    g_sorted.resize(n);
+    for (const IdxPair &p : *pairs) g_sorted[g_count[(size_t)p.ctx]++] = p;
+    pairs->swap(g_sorted);
+}
+
+// Validates the two lists and turns them into pairs.  `sort` (migration only): the pairs may
+// be handed to the kernel in another order than the caller's (option "sort_pairs").
+// `neighbours` (optional): whether at least half of the source blocks, in the order the
+// kernel gets them, follow their predecessor directly, i.e. the list is mostly runs of
+// adjacent blocks.
 int check_indices(const int64_t *src, const int64_t *dst, int64_t n, int64_t n_src, int64_t n_dst,
                   const char *src_name, const char *dst_name, std::vector<IdxPair> *pairs,
-                  bool *neighbours = nullptr)
+                  bool sort = false, bool *neighbours = nullptr)
 {
     if (n_dst > INT32_MAX || n_src > INT32_MAX)
         return fail(KVM_EINVAL, "pools of more than 2^31 blocks are not supported");
     g_seen.assign((size_t)((n_dst + 63) / 64), 0);
     pairs->resize((size_t)n);
     int64_t adjacent = 0;
+    bool ascending = true;
     for (int64_t i = 0; i < n; ++i) {
         const int64_t a = src[i], b = dst[i];
         if (a < 0 || a >= n_src)
@@ -848,6 +1012,16 @@ int check_indices(const int64_t *src, const int64_t *dst, int64_t n, int64_t n_s
         w |= bit;
         (*pairs)[(size_t)i] = IdxPair{(int32_t)a, (int32_t)b};
         if (i > 0 && a == src[i - 1] + 1) ++adjacent;
+        if (i > 0 && a < src[i - 1]) ascending = false;
+    }
+    // Sorting pays when the call names a large part of the source pool (measured: +4 % on
+    // calls of 800 of 1024 blocks whose rows are half read, +1 % on 1168 of 2048, nothing on
+    // 136 of 1024), and costs host time otherwise: a quarter of the pool is the line.
+    const int64_t mode = sort ? opt_sort_pairs.load() : 0;
+    if (!ascending && (mode == 2 || (mode == 1 && n >= 64 && 4 * n >= n_src))) {
+        sort_by_source(pairs, n_src);
+        adjacent = 0;
+        for (int64_t i = 1; i < n; ++i) adjacent += (*pairs)[(size_t)i].ctx == (*pairs)[(size_t)i - 1].ctx + 1;
     }
     if (neighbours) *neighbours = n > 1 && 2 * adjacent >= n - 1;
     return KVM_OK;
@@ -959,13 +1133,201 @@ int64_t swap_mode_for(const IdxPair *pairs, int64_t n, int64_t slab_bytes, int64
     return runs > 0 && (n * slab_bytes) / runs < opt_swap_kernel_below.load() ? 1 : 2;
 }
 
+// ---- memory handles and bindings
+
+// What a handle resolves to in this process.
+struct Resolved {
+    const char *ptr = nullptr;
+    int64_t nbytes = 0;
+    const char *map = nullptr;   // local base of the other process's allocation, null for a pool of this process
+};
+
+// Unmaps the mappings `doomed` selects, after dropping the pools bound through them and after
+// the device has finished whatever may still read them.  The caller holds g_reg_mu.
+template <typename Pred>
+int close_mappings(Pred doomed)
+{
+    bool any = false;
+    for (const Opened &o : g_opened) any = any || doomed(o);
+    if (!any) return KVM_OK;
+    int rc = KVM_OK;
+    std::unique_lock<std::shared_mutex> lock(g_mu);   // no migrate call is between its lookup and its launch
+    for (const Opened &o : g_opened) {
+        if (!doomed(o)) continue;
+        for (auto it = g_sources.begin(); it != g_sources.end();)
+            it = (it->second.map_k == o.local_base || it->second.map_v == o.local_base) ? g_sources.erase(it) : ++it;
+    }
+    if (hipDeviceSynchronize() != hipSuccess) {
+        (void)hipGetLastError();
+        rc = fail(KVM_EHIP, "the device did not become idle before a mapping was closed");
+    }
+    for (size_t i = 0; i < g_opened.size();) {
+        if (!doomed(g_opened[i])) {
+            ++i;
+            continue;
+        }
+        const hipError_t e = hipIpcCloseMemHandle(g_opened[i].local_base);
+        if (e != hipSuccess) {
+            (void)hipGetLastError();
+            rc = fail(KVM_EHIP, "hipIpcCloseMemHandle failed: %s", hipGetErrorString(e));
+        }
+        g_opened.erase(g_opened.begin() + (ptrdiff_t)i);
+    }
+    return rc;
+}
+
+// Mappings that no registered pool lies in any more (a binding was replaced, a registration
+// failed half way): they would keep the exporter's freed memory pinned.
+int close_unreferenced_mappings()
+{
+    std::vector<const char *> used;
+    {
+        std::shared_lock<std::shared_mutex> lock(g_mu);
+        for (const auto &kv : g_sources) {
+            if (kv.second.map_k) used.push_back(kv.second.map_k);
+            if (kv.second.map_v) used.push_back(kv.second.map_v);
+        }
+    }
+    return close_mappings([&used](const Opened &o) {
+        return std::find(used.begin(), used.end(), (const char *)o.local_base) == used.end();
+    });
+}
+
+// Resolves a handle to a pointer valid in this process, mapping the exporter's allocation
+// if it is another process's and not mapped yet.  The caller holds g_reg_mu.
+int open_handle(const int64_t *h, const char *what, Resolved *out)
+{
+    if (!h) return fail(KVM_EINVAL, "%s handle is null", what);
+    if (h[kHwMagic] != kHandleMagic || h[kHwCheck] != handle_check(h))
+        return fail(KVM_EHANDLE, "%s handle is not a kvmove memory handle", what);
+    if (h[kHwBytes] <= 0 || h[kHwPtr] == 0)
+        return fail(KVM_EHANDLE, "%s handle names no memory", what);
+    out->nbytes = h[kHwBytes];
+    out->map = nullptr;
+    if (is_own_handle(h)) {
+        out->ptr = (const char *)(uintptr_t)h[kHwPtr];
+        return KVM_OK;
+    }
+    if (!(h[kHwFlags] & kHandleHasIpc)) {
+        if (h[kHwAllocSize] >= KVM_IPC_MAX_ALLOC_BYTES)
+            return fail(KVM_EHANDLE,
+                        "%s handle of process %lld names a pool inside an allocation of %lld bytes; allocations of "
+                        "%lld bytes and more are not shared between processes",
+                        what, (long long)h[kHwPid], (long long)h[kHwAllocSize], (long long)KVM_IPC_MAX_ALLOC_BYTES);
+        return fail(KVM_EHANDLE, "%s handle of process %lld was not exported for other processes", what,
+                    (long long)h[kHwPid]);
+    }
+    const int64_t off = h[kHwPtr] - h[kHwAllocBase];
+    if (h[kHwAllocSize] <= 0 || h[kHwAllocSize] >= KVM_IPC_MAX_ALLOC_BYTES || off < 0 ||
+        off + h[kHwBytes] > h[kHwAllocSize])
+        return fail(KVM_EHANDLE, "%s handle of process %lld is inconsistent (pool at offset %lld, %lld bytes, in an "
+                    "allocation of %lld)", what, (long long)h[kHwPid], (long long)off, (long long)h[kHwBytes],
+                    (long long)h[kHwAllocSize]);
+    hipIpcMemHandle_t ipc;
+    memcpy(&ipc, &h[kHwIpc], sizeof ipc);
+    const int64_t serial = (int64_t)((uint64_t)h[kHwFlags] >> kHandleSerialShift);
+    for (const Opened &o : g_opened) {
+        if (o.pid != h[kHwPid] || o.nonce != h[kHwNonce] || o.remote_base != h[kHwAllocBase]) continue;
+        // The same allocation: its id matches, or -- where the exporter had no id to give -- it
+        // was mapped by this very registration call (a rank's K and V pools in one allocation).
+        // A mapping without an id is never trusted across calls: the exporter may have freed
+        // the memory and allocated anew at the same address.
+        if (serial != 0 ? o.serial == serial : (o.serial == 0 && o.opened_in == g_reg_call)) {
+            if (o.size != h[kHwAllocSize])
+                return fail(KVM_EHANDLE, "%s handle of process %lld says its allocation holds %lld bytes, the same "
+                            "allocation is open with %lld", what, (long long)h[kHwPid], (long long)h[kHwAllocSize],
+                            (long long)o.size);
+            out->ptr = o.local_base + off;
+            out->map = o.local_base;
+            return KVM_OK;
+        }
+        // The exporting process has made a new allocation at the old address (or may have): the
+        // old mapping and every pool bound through it are stale.
+        const char *stale = o.local_base;
+        if (int rc = close_mappings([stale](const Opened &x) { return x.local_base == stale; })) return rc;
+        break;
+    }
+    void *local = nullptr;
+    const hipError_t e = hipIpcOpenMemHandle(&local, ipc, hipIpcMemLazyEnablePeerAccess);
+    if (e != hipSuccess || !local) {
+        (void)hipGetLastError();
+        return fail(KVM_EHANDLE, "%s handle of process %lld could not be opened: %s", what, (long long)h[kHwPid],
+                    hipGetErrorString(e));
+    }
+    // The size in the handle is the exporter's word; where the runtime can tell how much it
+    // has mapped, a handle that claims more is refused before a kernel could run off the end.
+    const uint64_t mapped = extent_of(local);
+    if (mapped != 0 && mapped < (uint64_t)h[kHwAllocSize]) {
+        (void)hipIpcCloseMemHandle(local);
+        return fail(KVM_EHANDLE, "%s handle of process %lld says its allocation holds %lld bytes, the mapping holds %llu",
+                    what, (long long)h[kHwPid], (long long)h[kHwAllocSize], (unsigned long long)mapped);
+    }
+    g_opened.push_back(Opened{h[kHwPid], h[kHwNonce], h[kHwAllocBase], h[kHwAllocSize], serial, g_reg_call, (char *)local});
+    out->ptr = (char *)local + off;
+    out->map = (char *)local;
+    return KVM_OK;
+}
+
+int check_source_args(int32_t ctx_pp_size, int32_t ctx_tp_size, int32_t pp_rank, int32_t tp_rank,
+                             int64_t num_layers, int64_t num_kv_heads, const void *k_base, const void *v_base,
+                             int64_t nbytes_each)
+{
+    if (!k_base || !v_base || nbytes_each <= 0)
+        return fail(KVM_EINVAL, "kvm_register_source: null pool or non-positive size");
+    if (ctx_pp_size <= 0 || ctx_tp_size <= 0 || pp_rank < 0 || pp_rank >= ctx_pp_size || tp_rank < 0 ||
+        tp_rank >= ctx_tp_size)
+        return fail(KVM_EINVAL, "context rank (pp %d, tp %d) outside (pp %d, tp %d)", pp_rank, tp_rank,
+                    ctx_pp_size, ctx_tp_size);
+    if (num_layers <= 0 || num_kv_heads <= 0 || num_layers % ctx_pp_size || num_kv_heads % ctx_tp_size)
+        return fail(KVM_EINVAL, "L %lld / H %lld do not split over pp %d / tp %d", (long long)num_layers,
+                    (long long)num_kv_heads, ctx_pp_size, ctx_tp_size);
+    return KVM_OK;
+}
+
+// A pool of this process: device memory whose allocation holds the bytes it claims.
+int check_local_pool(const void *p, int64_t nbytes, const char *what, int *device)
+{
+    if (int rc = device_of(p, what, device)) return rc;
+    return check_extent(p, (uint64_t)nbytes, extent_of(p), what);
+}
+
+// Binds one context rank's pools.  Pools that were resolved through a mapping (map != null)
+// are device memory of the size their handle states: open_handle has checked that the pool
+// lies inside the mapping, and the runtime's own queries may not know a mapping as an
+// allocation; every other pointer is checked here.  The caller holds g_reg_mu.
+int bind_source(int32_t ctx_pp_size, int32_t ctx_tp_size, int32_t pp_rank, int32_t tp_rank,
+                       int64_t num_layers, int64_t num_kv_heads, const Resolved &k, const Resolved &v,
+                       int64_t ctx_instance)
+{
+    if (k.nbytes != v.nbytes)
+        return fail(KVM_EMISMATCH, "K pool (%lld bytes) and V pool (%lld bytes) differ", (long long)k.nbytes,
+                    (long long)v.nbytes);
+    if (int rc = check_source_args(ctx_pp_size, ctx_tp_size, pp_rank, tp_rank, num_layers, num_kv_heads, k.ptr,
+                                   v.ptr, k.nbytes))
+        return rc;
+    int dk = -1, dv = -1;
+    if (!k.map)
+        if (int rc = check_local_pool(k.ptr, k.nbytes, "context K pool", &dk)) return rc;
+    if (!v.map)
+        if (int rc = check_local_pool(v.ptr, v.nbytes, "context V pool", &dv)) return rc;
+    if (dk >= 0 && dv >= 0 && dk != dv) return fail(KVM_EINVAL, "context K and V pools sit on different devices");
+    const Source s{ctx_pp_size, ctx_tp_size, num_layers, num_kv_heads, k.ptr, v.ptr, k.nbytes, k.map, v.map};
+    std::unique_lock<std::shared_mutex> lock(g_mu);
+    g_sources[SourceKey{ctx_instance, pp_rank, tp_rank}] = s;
+    return KVM_OK;
+}
+
+// Whether a call's index pairs fit the packed table: every index is below its pool's block
+// count, so pools of at most 65536 blocks make every index fit 16 bits.
+bool fits_packed(int64_t n_src, int64_t n_dst) { return n_src <= 65536 && n_dst <= 65536; }
+
 }  // namespace
 
 // ------------------------------------------------------------------------- C ABI
 
 extern "C" {
 
-int kvm_version(void) { return 100; }
+int kvm_version(void) { return KVM_ABI_MAJOR * 10000 + 0 * 100 + 0; }
 
 const char *kvm_last_error(void) { return g_err.c_str(); }
 
@@ -974,14 +1336,20 @@ int kvm_set_option(const char *name, int64_t value)
     std::atomic<int64_t> *o = find_opt(name);
     if (!o) return fail(KVM_EINVAL, "unknown option '%s'", name ? name : "(null)");
     bool ok = true;
-    if (o == &opt_tile_bytes) ok = value == 0 || (value >= 1024 && value <= (1 << 26) && (value & (value - 1)) == 0);
-    else if (o == &opt_threads) ok = value == 64 || value == 128 || value == 256 || value == 512 || value == 1024;
-    else if (o == &opt_unroll) ok = value == 1 || value == 2 || value == 4 || value == 8 || value == 16;
-    else if (o == &opt_swap_wgs || o == &opt_swap_wgs_in) ok = value >= 1 && value <= 4096;
-    else if (o == &opt_lds_pad) ok = value >= 0 && value <= 65536;
+    if (o == &opt_swap_wgs || o == &opt_swap_wgs_in) ok = value >= 1 && value <= 4096;
     else if (o == &opt_xcd_map) ok = value >= 0 && value <= 3;
     else if (o == &opt_swap_mode) ok = value >= 0 && value <= 3;
     else if (o == &opt_swap_kernel_below) ok = value >= 0 && value <= (1ll << 32);
+    else if (o == &opt_sort_pairs) ok = value >= 0 && value <= 2;
+#ifdef KVM_EXPLORE
+    else if (o == &opt_tile_bytes) ok = value == 0 || (value >= 1024 && value <= (1 << 26) && (value & (value - 1)) == 0);
+    else if (o == &opt_threads) ok = value == 64 || value == 128 || value == 256 || value == 512 || value == 1024;
+    else if (o == &opt_unroll) ok = value == 1 || value == 2 || value == 4 || value == 8 || value == 16;
+    else if (o == &opt_lds_pad) ok = value >= 0 && value <= 65536;
+    else if (o == &opt_max_pairs) ok = value >= 1 && value <= kMaxIdxPacked;
+    else if (o == &opt_swap_threads) ok = value >= 64 && value <= 1024;
+    else if (o == &opt_swap_unroll) ok = value >= 1 && value <= 8;
+#endif
     else ok = value == 0 || value == 1;
     if (!ok) return fail(KVM_EINVAL, "value %lld is not valid for option '%s'", (long long)value, name);
     o->store(value);
@@ -1008,6 +1376,7 @@ int kvm_get_mem_handle(const void *dev_ptr, int64_t nbytes, int64_t *out_handle)
     h[kHwDevice] = dev;
     h[kHwPtr] = (int64_t)(uintptr_t)dev_ptr;
     h[kHwBytes] = nbytes;
+    h[kHwNonce] = process_nonce();
     // The IPC handle names a whole allocation, so the pool travels as (allocation, offset).
     hipDeviceptr_t base = nullptr;
     size_t size = 0;
@@ -1040,116 +1409,19 @@ int kvm_get_mem_handle(const void *dev_ptr, int64_t nbytes, int64_t *out_handle)
     return KVM_OK;
 }
 
-// Resolves a handle to a pointer valid in this process.  *map = local base of the other
-// process's allocation when the handle had to be opened, null for one of this process's.
-// The caller holds g_mu.
-static int open_handle(const int64_t *h, const char *what, const char **ptr, int64_t *nbytes, const char **map)
-{
-    if (!h) return fail(KVM_EINVAL, "%s handle is null", what);
-    if (h[kHwMagic] != kHandleMagic || h[kHwCheck] != handle_check(h))
-        return fail(KVM_EHANDLE, "%s handle is not a kvmove memory handle", what);
-    if (h[kHwBytes] <= 0 || h[kHwPtr] == 0)
-        return fail(KVM_EHANDLE, "%s handle names no memory", what);
-    *nbytes = h[kHwBytes];
-    *map = nullptr;
-    if (h[kHwPid] == (int64_t)getpid()) {
-        *ptr = (const char *)(uintptr_t)h[kHwPtr];
-        return KVM_OK;
-    }
-    if (!(h[kHwFlags] & kHandleHasIpc)) {
-        if (h[kHwAllocSize] >= KVM_IPC_MAX_ALLOC_BYTES)
-            return fail(KVM_EHANDLE,
-                        "%s handle of process %lld names a pool inside an allocation of %lld bytes; allocations of "
-                        "%lld bytes and more are not shared between processes",
-                        what, (long long)h[kHwPid], (long long)h[kHwAllocSize], (long long)KVM_IPC_MAX_ALLOC_BYTES);
-        return fail(KVM_EHANDLE, "%s handle of process %lld was not exported for other processes", what,
-                    (long long)h[kHwPid]);
-    }
-    const int64_t off = h[kHwPtr] - h[kHwAllocBase];
-    if (h[kHwAllocSize] <= 0 || h[kHwAllocSize] >= KVM_IPC_MAX_ALLOC_BYTES || off < 0 ||
-        off + h[kHwBytes] > h[kHwAllocSize])
-        return fail(KVM_EHANDLE, "%s handle of process %lld is inconsistent (pool at offset %lld, %lld bytes, in an "
-                    "allocation of %lld)", what, (long long)h[kHwPid], (long long)off, (long long)h[kHwBytes],
-                    (long long)h[kHwAllocSize]);
-    hipIpcMemHandle_t ipc;
-    memcpy(&ipc, &h[kHwIpc], sizeof ipc);
-    const int64_t serial = (int64_t)((uint64_t)h[kHwFlags] >> kHandleSerialShift);
-    for (size_t i = 0; i < g_opened.size(); ++i) {
-        Opened &o = g_opened[i];
-        if (o.pid != h[kHwPid] || o.remote_base != h[kHwAllocBase]) continue;
-        if (o.serial == serial) {
-            if (o.size != h[kHwAllocSize])
-                return fail(KVM_EHANDLE, "%s handle of process %lld says its allocation holds %lld bytes, the same "
-                            "allocation is open with %lld", what, (long long)h[kHwPid], (long long)h[kHwAllocSize],
-                            (long long)o.size);
-            *ptr = o.local_base + off;
-            *map = o.local_base;
-            return KVM_OK;
-        }
-        // The exporting process has made a new allocation at the old address: the old
-        // mapping and every pool bound through it are stale.
-        KVM_HIP(hipDeviceSynchronize());
-        for (auto it = g_sources.begin(); it != g_sources.end();)
-            it = (it->second.map_k == o.local_base || it->second.map_v == o.local_base) ? g_sources.erase(it) : ++it;
-        (void)hipIpcCloseMemHandle(o.local_base);
-        g_opened.erase(g_opened.begin() + (ptrdiff_t)i);
-        break;
-    }
-    void *local = nullptr;
-    const hipError_t e = hipIpcOpenMemHandle(&local, ipc, hipIpcMemLazyEnablePeerAccess);
-    if (e != hipSuccess || !local) {
-        (void)hipGetLastError();
-        return fail(KVM_EHANDLE, "%s handle of process %lld could not be opened: %s", what, (long long)h[kHwPid],
-                    hipGetErrorString(e));
-    }
-    // The size in the handle is the exporter's word; where the runtime can tell how much it
-    // has mapped, a handle that claims more is refused before a kernel could run off the end.
-    const uint64_t mapped = extent_of(local);
-    if (mapped != 0 && mapped < (uint64_t)h[kHwAllocSize]) {
-        (void)hipIpcCloseMemHandle(local);
-        return fail(KVM_EHANDLE, "%s handle of process %lld says its allocation holds %lld bytes, the mapping holds %llu",
-                    what, (long long)h[kHwPid], (long long)h[kHwAllocSize], (unsigned long long)mapped);
-    }
-    g_opened.push_back(Opened{h[kHwPid], h[kHwAllocBase], h[kHwAllocSize], serial, (char *)local});
-    *ptr = (char *)local + off;
-    *map = (char *)local;
-    return KVM_OK;
-}
-
-static int check_source_args(int32_t ctx_pp_size, int32_t ctx_tp_size, int32_t pp_rank, int32_t tp_rank,
-                             int64_t num_layers, int64_t num_kv_heads, const void *k_base, const void *v_base,
-                             int64_t nbytes_each)
-{
-    if (!k_base || !v_base || nbytes_each <= 0)
-        return fail(KVM_EINVAL, "kvm_register_source: null pool or non-positive size");
-    if (ctx_pp_size <= 0 || ctx_tp_size <= 0 || pp_rank < 0 || pp_rank >= ctx_pp_size || tp_rank < 0 ||
-        tp_rank >= ctx_tp_size)
-        return fail(KVM_EINVAL, "context rank (pp %d, tp %d) outside (pp %d, tp %d)", pp_rank, tp_rank,
-                    ctx_pp_size, ctx_tp_size);
-    if (num_layers <= 0 || num_kv_heads <= 0 || num_layers % ctx_pp_size || num_kv_heads % ctx_tp_size)
-        return fail(KVM_EINVAL, "L %lld / H %lld do not split over pp %d / tp %d", (long long)num_layers,
-                    (long long)num_kv_heads, ctx_pp_size, ctx_tp_size);
-    return KVM_OK;
-}
-
 int kvm_register_source(int32_t ctx_pp_size, int32_t ctx_tp_size, int32_t pp_rank, int32_t tp_rank,
                         int64_t num_layers, int64_t num_kv_heads, const void *k_base,
                         const void *v_base, int64_t nbytes_each, int64_t ctx_instance)
 {
-    if (int rc = check_source_args(ctx_pp_size, ctx_tp_size, pp_rank, tp_rank, num_layers, num_kv_heads, k_base,
-                                   v_base, nbytes_each))
+    Resolved k, v;
+    k.ptr = (const char *)k_base;
+    v.ptr = (const char *)v_base;
+    k.nbytes = v.nbytes = nbytes_each;
+    std::lock_guard<std::mutex> reg(g_reg_mu);
+    ++g_reg_call;
+    if (int rc = bind_source(ctx_pp_size, ctx_tp_size, pp_rank, tp_rank, num_layers, num_kv_heads, k, v, ctx_instance))
         return rc;
-    int dk = 0, dv = 0;
-    if (int rc = device_of(k_base, "context K pool", &dk)) return rc;
-    if (int rc = device_of(v_base, "context V pool", &dv)) return rc;
-    if (dk != dv) return fail(KVM_EINVAL, "context K and V pools sit on different devices");
-    if (int rc = check_extent(k_base, (uint64_t)nbytes_each, extent_of(k_base), "context K pool")) return rc;
-    if (int rc = check_extent(v_base, (uint64_t)nbytes_each, extent_of(v_base), "context V pool")) return rc;
-    Source s{ctx_pp_size, ctx_tp_size, num_layers, num_kv_heads, (const char *)k_base,
-             (const char *)v_base, nbytes_each, nullptr, nullptr};
-    std::lock_guard<std::mutex> lock(g_mu);
-    g_sources[SourceKey{ctx_instance, pp_rank, tp_rank}] = s;
-    return KVM_OK;
+    return close_unreferenced_mappings();   // the binding this one replaced may have been the last in a mapping
 }
 
 int kvm_register_mem_handle(const int64_t *k_handle, const int64_t *v_handle, int64_t num_layers,
@@ -1170,85 +1442,65 @@ int kvm_register_mem_handle(const int64_t *k_handle, const int64_t *v_handle, in
             return fail(KVM_EINVAL, "context parallel config [%lld,%lld,%lld,%lld] is malformed",
                         (long long)context_pc[0], (long long)context_pc[1], (long long)context_pc[2],
                         (long long)context_pc[3]);
-    // Handles of this process take the same road as raw pointers.
-    if (k_handle[kHwMagic] == kHandleMagic && v_handle[kHwMagic] == kHandleMagic &&
-        k_handle[kHwPid] == (int64_t)getpid() && v_handle[kHwPid] == (int64_t)getpid()) {
-        const char *k = nullptr, *v = nullptr, *mk = nullptr, *mv = nullptr;
-        int64_t kb = 0, vb = 0;
-        if (int rc = open_handle(k_handle, "K", &k, &kb, &mk)) return rc;
-        if (int rc = open_handle(v_handle, "V", &v, &vb, &mv)) return rc;
-        if (kb != vb) return fail(KVM_EMISMATCH, "K pool (%lld bytes) and V pool (%lld bytes) differ",
-                                  (long long)kb, (long long)vb);
-        return kvm_register_source((int32_t)context_pc[2], (int32_t)context_pc[0], (int32_t)context_pc[3],
-                                   (int32_t)context_pc[1], num_layers, num_kv_heads, k, v, kb, ctx_instance);
-    }
-    std::lock_guard<std::mutex> lock(g_mu);
-    const char *k = nullptr, *v = nullptr, *mk = nullptr, *mv = nullptr;
-    int64_t kb = 0, vb = 0;
-    if (int rc = open_handle(k_handle, "K", &k, &kb, &mk)) return rc;
-    if (int rc = open_handle(v_handle, "V", &v, &vb, &mv)) return rc;
-    if (kb != vb) return fail(KVM_EMISMATCH, "K pool (%lld bytes) and V pool (%lld bytes) differ",
-                              (long long)kb, (long long)vb);
-    if (int rc = check_source_args((int32_t)context_pc[2], (int32_t)context_pc[0], (int32_t)context_pc[3],
-                                   (int32_t)context_pc[1], num_layers, num_kv_heads, k, v, kb))
-        return rc;
-    // A mapped allocation is device memory of the size its handle states: open_handle has
-    // checked that the pool lies inside it, and the runtime's own queries may not know the
-    // mapping as an allocation.
-    Source s{(int32_t)context_pc[2], (int32_t)context_pc[0], num_layers, num_kv_heads, k, v, kb, mk, mv};
-    g_sources[SourceKey{ctx_instance, (int32_t)context_pc[3], (int32_t)context_pc[1]}] = s;
-    return KVM_OK;
+    std::lock_guard<std::mutex> reg(g_reg_mu);
+    ++g_reg_call;
+    Resolved k, v;
+    int rc = open_handle(k_handle, "K", &k);
+    if (rc == KVM_OK) rc = open_handle(v_handle, "V", &v);
+    if (rc == KVM_OK)
+        rc = bind_source((int32_t)context_pc[2], (int32_t)context_pc[0], (int32_t)context_pc[3],
+                         (int32_t)context_pc[1], num_layers, num_kv_heads, k, v, ctx_instance);
+    // Whatever this call mapped and did not bind (the V handle failed after the K handle had
+    // opened, the pools disagreed), and whatever the replaced binding leaves unused, goes.
+    const std::string text = g_err;
+    const int rc_close = close_unreferenced_mappings();
+    if (rc != KVM_OK) g_err = text;
+    return rc != KVM_OK ? rc : rc_close;
 }
 
 int kvm_reset(void)
 {
-    std::lock_guard<std::mutex> lock(g_mu);
-    g_sources.clear();
-    int rc = KVM_OK;
-    if (!g_opened.empty()) {
-        // kernels in flight may still read the mappings
-        if (hipDeviceSynchronize() != hipSuccess) {
-            (void)hipGetLastError();
-            rc = fail(KVM_EHIP, "kvm_reset: the device did not become idle");
-        }
-        for (Opened &o : g_opened) {
-            const hipError_t e = hipIpcCloseMemHandle(o.local_base);
-            if (e != hipSuccess) {
-                (void)hipGetLastError();
-                rc = fail(KVM_EHIP, "hipIpcCloseMemHandle failed: %s", hipGetErrorString(e));
-            }
-        }
-        g_opened.clear();
+    std::lock_guard<std::mutex> reg(g_reg_mu);
+    {
+        std::unique_lock<std::shared_mutex> lock(g_mu);
+        g_sources.clear();
     }
-    return rc;
+    // kernels in flight may still read the mappings: close_mappings waits for the device first
+    return close_mappings([](const Opened &) { return true; });
 }
 
 int64_t kvm_opened_handles(void)
 {
-    std::lock_guard<std::mutex> lock(g_mu);
+    std::lock_guard<std::mutex> reg(g_reg_mu);
     return (int64_t)g_opened.size();
 }
 
-int kvm_migrate_plan(const KvmGeom *geom, int64_t n, const void *dst_k, const void *dst_v, int64_t out[8])
+int kvm_migrate_plan(const KvmGeom *geom, int64_t n, const void *dst_k, const void *dst_v, int64_t dst_num_blocks,
+                     int64_t out[10])
 {
     if (!out) return fail(KVM_EINVAL, "out is null");
     if (n < 0) return fail(KVM_EINVAL, "n is negative");
+    const bool arithmetic_only = !dst_k && !dst_v;
     Plan plan;
-    if (int rc = build_plan(geom, dst_k, dst_v, &plan, !dst_k && !dst_v)) return rc;
-    int64_t launches = 0, wgs = 0, max_items = 0;
-    int threads = 0;
-    bool simple = false;
-    if (int rc = launch_copy(plan.segs, nullptr, n, nullptr, nullptr, plan.dst_block_stride, plan.vec,
-                             nullptr, &launches, &wgs, &threads, 0, &simple, &max_items))
+    std::shared_lock<std::shared_mutex> lock(g_mu);
+    if (int rc = build_plan(geom, dst_k, dst_v, &plan, arithmetic_only)) return rc;
+    // pools that are not registered count as being as large as the destination pool is said to be
+    const int64_t n_src = arithmetic_only ? dst_num_blocks : plan.min_src_blocks;
+    const bool packed = dst_num_blocks > 0 && fits_packed(n_src, dst_num_blocks);
+    CopyShape shape;
+    if (int rc = launch_copy(plan.segs, nullptr, n, packed, nullptr, nullptr, plan.dst_block_stride, plan.vec,
+                             nullptr, &shape))
         return rc;
-    out[0] = wgs;
-    out[1] = threads;
+    out[0] = shape.wgs_per_block;
+    out[1] = shape.threads;
     out[2] = plan.vec;
     out[3] = (int64_t)plan.segs.size();
-    out[4] = launches;
+    out[4] = shape.launches;
     out[5] = plan.payload_per_block;
-    out[6] = simple ? 1 : 0;
-    out[7] = max_items;
+    out[6] = shape.simple ? 1 : 0;
+    out[7] = shape.max_items;
+    out[8] = shape.unroll;
+    out[9] = shape.pairs_per_launch;
     return KVM_OK;
 }
 
@@ -1261,6 +1513,8 @@ int kvm_migrate(const KvmGeom *geom, const int64_t *ctx_idx, const int64_t *dec_
     if (n > 0 && (!ctx_idx || !dec_idx)) return fail(KVM_EINVAL, "index list is null");
     if (n == 0) return check_geom(geom);   // an empty list moves nothing, whatever is registered
     Plan plan;
+    // held until the last launch is enqueued: no registration can unmap a pool in between
+    std::shared_lock<std::shared_mutex> lock(g_mu);
     if (int rc = build_plan(geom, dst_k, dst_v, &plan)) return rc;
     const uint64_t dst_bytes = (uint64_t)dst_num_blocks * plan.dst_block_stride;
     if (int rc = checked_pool(dst_k, dst_bytes, true, "decoding K pool")) return rc;
@@ -1268,15 +1522,15 @@ int kvm_migrate(const KvmGeom *geom, const int64_t *ctx_idx, const int64_t *dec_
     std::vector<IdxPair> pairs;
     bool neighbours = false;
     if (int rc = check_indices(ctx_idx, dec_idx, n, plan.min_src_blocks, dst_num_blocks,
-                               "context_block_indexes", "decoding_block_indexes", &pairs, &neighbours))
+                               "context_block_indexes", "decoding_block_indexes", &pairs, true, &neighbours))
         return rc;
-    return launch_copy(std::move(plan.segs), pairs.data(), n, (char *)dst_k, (char *)dst_v,
-                       plan.dst_block_stride, plan.vec, (hipStream_t)stream, nullptr, nullptr, nullptr, 0, nullptr,
-                       nullptr, neighbours);
+    return launch_copy(std::move(plan.segs), pairs.data(), n, fits_packed(plan.min_src_blocks, dst_num_blocks),
+                       (char *)dst_k, (char *)dst_v, plan.dst_block_stride, plan.vec, (hipStream_t)stream, nullptr, 0,
+                       neighbours);
 }
 
 int kvm_swap_plan(const int64_t *src_ids, const int64_t *dst_ids, int64_t n, int64_t slab_bytes, int is_swap_in,
-                  int64_t out[4])
+                  int64_t n_gpu_blocks, int64_t n_host_blocks, int64_t out[4])
 {
     if (!out) return fail(KVM_EINVAL, "out is null");
     if (n < 0 || (n > 0 && (!src_ids || !dst_ids))) return fail(KVM_EINVAL, "bad index lists");
@@ -1292,7 +1546,9 @@ int kvm_swap_plan(const int64_t *src_ids, const int64_t *dst_ids, int64_t n, int
     const int64_t mode = swap_mode_for(pairs.data(), n, slab_bytes, &runs);
     out[0] = mode;
     out[1] = runs;
-    out[2] = mode == 1 ? (n + kMaxIdx - 1) / kMaxIdx : 0;
+    const int64_t per_launch = n_gpu_blocks > 0 && n_host_blocks > 0 && fits_packed(n_gpu_blocks, n_host_blocks) &&
+                                       tune_packed() ? kMaxIdxPacked : kMaxIdx;
+    out[2] = mode == 1 ? (n + per_launch - 1) / per_launch : 0;
     out[3] = mode == 1 ? (is_swap_in ? opt_swap_wgs_in.load() : opt_swap_wgs.load()) : 0;
     return KVM_OK;
 }
@@ -1354,8 +1610,9 @@ int kvm_swap(const int64_t *src_ids, const int64_t *dst_ids, int64_t n, int is_s
         s.n_rows = 1;
         const int vec = vec_width((uint64_t)slab_bytes | (uintptr_t)src_k | (uintptr_t)src_v |
                                   (uintptr_t)dst_k | (uintptr_t)dst_v);
-        return launch_copy({s}, pairs.data(), n, dst_k, dst_v, (uint64_t)slab_bytes, vec, st, nullptr,
-                           nullptr, nullptr, (int)(is_swap_in ? opt_swap_wgs_in.load() : opt_swap_wgs.load()));
+        return launch_copy({s}, pairs.data(), n, fits_packed(n_gpu_blocks, n_host_blocks), dst_k, dst_v,
+                           (uint64_t)slab_bytes, vec, st, nullptr,
+                           (int)(is_swap_in ? opt_swap_wgs_in.load() : opt_swap_wgs.load()));
     }
 
     // hipMemcpyAsync per run of blocks that are consecutive on both sides.  In mode 2 the V
@@ -1421,9 +1678,8 @@ int kvm_copy_plain(void *dst, const void *src, int64_t nbytes, void *stream)
         s.n_rows = 1;
         std::vector<IdxPair> pairs((size_t)half_chunks);
         for (int64_t i = 0; i < half_chunks; ++i) pairs[(size_t)i] = IdxPair{(int32_t)i, (int32_t)i};
-        if (int rc = launch_copy({s}, pairs.data(), half_chunks, (char *)dst,
-                                 (char *)dst + half_chunks * chunk, (uint64_t)chunk, vec,
-                                 (hipStream_t)stream, nullptr, nullptr, nullptr))
+        if (int rc = launch_copy({s}, pairs.data(), half_chunks, fits_packed(half_chunks, half_chunks), (char *)dst,
+                                 (char *)dst + half_chunks * chunk, (uint64_t)chunk, vec, (hipStream_t)stream))
             return rc;
         done = 2 * half_chunks * chunk;
     }

@@ -162,6 +162,9 @@ void swap(std::vector<int64_t> source_block_ids, std::vector<int64_t> target_blo
 
 KVM_TORCH_LIBRARY(KVM_MIGRATION_NS, m)
 {
+    // structs, handles and signatures are only what this file was compiled against within one major version
+    TORCH_CHECK(kvm_version() / 10000 == KVM_ABI_MAJOR, "libkvmove.so is version ", kvm_version(),
+                ", this op library was built for major version ", KVM_ABI_MAJOR);
     m.def("get_ipc_mem_handle(Tensor t) -> int[]", get_ipc_mem_handle);
     m.def("register_ipc_mem_handle(int[] k_handle, int[] v_handle, int num_layers, int num_heads, "
           "int[] context_parallel_config, int[] decoding_parallel_config) -> ()",

@@ -35,15 +35,26 @@ def _require_gpu() -> None:
 
 class MigrationMark:
     """Stands for "the copies enqueued on ``stream`` so far" with the interface of an event
-    (``wait``, ``synchronize``, ``query``).  The HIP event behind it is only recorded when
-    somebody needs one: work that follows on the same stream is behind the copies by stream
-    order alone, and that is the common case (one worker thread, one current stream), where
-    an eager event per migrated request would be two runtime calls that order nothing.  An
-    event recorded late covers the copies all the same (and whatever the stream got since)."""
+    (``wait``, ``synchronize``, ``query``).  On the device's default stream the HIP event
+    behind it is only recorded when somebody needs one: work that follows on the same stream
+    is behind the copies by stream order alone, and that is the common case (one worker
+    thread, one current stream), where an eager event per migrated request would be two
+    runtime calls that order nothing.  An event recorded late covers the copies all the same,
+    and whatever the stream got since -- which is why a mark made on any OTHER stream records
+    at once (``eager``): a worker that migrates on a stream of its own has other streams
+    beside it, and one of them waiting on a late event would also wait for everything the
+    migration's stream was given after the copies (a long decoding step, say)."""
 
-    def __init__(self, stream: torch.cuda.Stream):
+    def __init__(self, stream: torch.cuda.Stream, eager: bool = False):
         self.stream = stream
         self._event: Optional[torch.cuda.Event] = None
+        if eager:
+            self._recorded()
+
+    @property
+    def pending(self) -> bool:
+        """No event has been recorded yet: the mark still stands for everything on its stream."""
+        return self._event is None
 
     def _recorded(self) -> torch.cuda.Event:
         if self._event is None:
@@ -81,6 +92,10 @@ class Worker:
         self.forward = forward
         self.device = torch.device("cuda:0")
         torch.cuda.set_device(self.device)
+        self._default_stream = torch.cuda.default_stream(self.device)
+        # the overloads, resolved once: a lookup through torch.ops per call costs microseconds
+        self._migrate_op = torch.ops.block_migration_ops.migrate_blocks_from.default
+        self._swap_op = torch.ops.swapping_ops.swap.default
 
         self.k_cache: Optional[torch.Tensor] = None   # [blocks, layers_local, kv_heads_local, B, D] on HBM
         self.v_cache: Optional[torch.Tensor] = None
@@ -189,7 +204,7 @@ class Worker:
                        decoding_block_indexes: List[int], context_instance: int = 0) -> None:
         """Pull this rank's share of the listed context blocks into its own pools, on the
         current stream, without waiting for the GPU (reference worker.py:250-267)."""
-        torch.ops.block_migration_ops.migrate_blocks_from(
+        self._migrate_op(
             context_instance,
             context_parallel_config.pipeline_parallel_size,
             context_parallel_config.tensor_parallel_size,
@@ -202,7 +217,11 @@ class Worker:
             self.k_cache,
             self.v_cache,
         )
-        self.latest_migrate_event = MigrationMark(self._current_stream())
+        stream = self._current_stream()
+        mark = self.latest_migrate_event
+        # a mark on the same stream that nobody has asked for an event yet stands for these copies too
+        if mark is None or not mark.pending or mark.stream != stream:
+            self.latest_migrate_event = MigrationMark(stream, eager=stream != self._default_stream)
 
     def wait_stream_for_migration(self, event: Optional[MigrationMark]) -> None:
         """Called on a *context* worker: work it enqueues from now on (the next prefill that
@@ -225,8 +244,8 @@ class Worker:
             if previous is not None:
                 previous.wait(stream)   # the request's earlier swap, possibly on the other stream
         with torch.cuda.stream(stream):
-            torch.ops.swapping_ops.swap(source_block_ids, target_block_ids, is_swap_in,
-                                        self.k_cache, self.v_cache, self.k_swap, self.v_swap)
+            self._swap_op(source_block_ids, target_block_ids, is_swap_in,
+                          self.k_cache, self.v_cache, self.k_swap, self.v_swap)
         event = torch.cuda.Event()
         event.record(stream)
         for request_id in request_ids:

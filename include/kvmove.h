@@ -42,7 +42,12 @@ extern "C" {
 #define KVM_EHANDLE (-6)    /* memory handle is malformed, or cannot be opened in this process */
 #define KVM_EMISMATCH (-7)  /* registered pools disagree with the call's geometry */
 
-#define KVM_HANDLE_WORDS 17 /* int64 words in a memory handle */
+#define KVM_HANDLE_WORDS 18 /* int64 words in a memory handle */
+
+/* Major version of this interface: kvm_version() / 10000.  It changes whenever a struct, a
+ * handle or a signature below changes shape; a caller compiled against another major version
+ * must not call anything but kvm_version() and kvm_last_error(). */
+#define KVM_ABI_MAJOR 1
 
 /* Device allocations of this size and above are not exported to other processes: the
  * handle of such a pool still works inside the process that made it. */
@@ -67,7 +72,8 @@ typedef struct KvmGeom {
                               one, as in the reference, where a decoding worker has one) */
 } KvmGeom;
 
-/* Library version: major*10000 + minor*100 + patch. */
+/* Library version: major*10000 + minor*100 + patch; the major part is KVM_ABI_MAJOR of the
+ * header the library was built from. */
 int kvm_version(void);
 
 /* Text of the last error on the calling thread ("" if none). */
@@ -76,10 +82,11 @@ const char *kvm_last_error(void);
 /*
  * Replaces torch.ops.block_migration_ops.get_ipc_mem_handle(tensor)
  * (distserve/worker.py:133-134).  Writes an opaque KVM_HANDLE_WORDS-word handle naming
- * the device memory [dev_ptr, dev_ptr + nbytes): the exporting process, the pointer, and a
- * hipIpcMemHandle_t of the device allocation that holds it together with the pool's offset
- * inside that allocation (a pool may be a piece of a larger allocation, as with torch's
- * caching allocator).  The words are plain data: send them to the decoding worker by any
+ * the device memory [dev_ptr, dev_ptr + nbytes): the exporting process (its pid and a random
+ * word it drew at start, so that two processes with one pid in different pid namespaces are
+ * told apart), the pointer, and a hipIpcMemHandle_t of the device allocation that holds it
+ * together with the pool's offset inside that allocation (a pool may be a piece of a larger
+ * allocation, as with torch's caching allocator).  The words are plain data: send them to the decoding worker by any
  * means.  Inside the exporting process the handle resolves to the pointer itself (a
  * process cannot open its own IPC handle); in another process registration maps the
  * allocation with hipIpcOpenMemHandle.  An allocation of KVM_IPC_MAX_ALLOC_BYTES or more,
@@ -96,10 +103,14 @@ int kvm_get_mem_handle(const void *dev_ptr, int64_t nbytes, int64_t *out_handle)
  * context_pc / decoding_pc are [tp_size, tp_rank, pp_size, pp_rank]
  * (distserve/config.py:57-63).  Registering the same rank again replaces the binding.
  * Handles made by another process are opened here (hipIpcOpenMemHandle, once per
- * allocation and process, however many pools lie in it) and stay mapped until kvm_reset.
+ * allocation and process, however many pools lie in it) and stay mapped while a bound pool
+ * lies in them (a mapping whose last pool was re-bound elsewhere is closed by the
+ * registration that re-bound it, after the device has gone idle) or until kvm_reset.
  * A handle carries the exporting runtime's id of its allocation: when the exporter has
  * freed its pools and allocated new ones, handles exported afterwards replace the stale
- * mapping (and drop the pools bound through it) even where an address recurs.
+ * mapping (and drop the pools bound through it) even where an address recurs; a handle
+ * whose exporter had no id to give is mapped anew by every registration call.  A call that
+ * fails leaves nothing mapped that it mapped itself.
  * ctx_instance (no counterpart in the reference, whose decoding worker serves a single
  * context instance) keeps the pools of several context instances apart in one process:
  * bindings are keyed by (ctx_instance, pp_rank, tp_rank), and a migrate call reads the
@@ -159,43 +170,44 @@ int kvm_swap(const int64_t *src_ids, const int64_t *dst_ids, int64_t n, int is_s
 int kvm_copy_plain(void *dst, const void *src, int64_t nbytes, void *stream);
 
 /*
- * Tuning knobs (no counterpart in the reference).  Names:
- *   "tile_bytes"     payload bytes one workgroup moves per pool kind: 0 (default) = exactly
- *                    what its lanes hold in flight, threads*unroll*16 ("one shot"), or a
- *                    power of two >= 1024
- *   "threads"        workgroup size: 64, 128, 256, 512 or 1024
- *   "unroll"         16-byte vectors in flight per lane: 1, 2, 4, 8 or 16
- *   "wave_contig"    1 = a wave's vectors are adjacent in memory, 0 = one pass apart
- *   "lds_pad"        bytes of LDS requested per workgroup only to limit occupancy (0..65536)
+ * Options (no counterpart in the reference), process-wide.  Names:
  *   "xcd_map"        how workgroup ids map to work: 0 = in order, 1 (default) = chosen per call:
  *                    in order when at least half of the call's context blocks follow their
  *                    predecessor in the list directly (neighbouring blocks), else each XCD walks
  *                    contiguous chunks (an eighth of a block when that is >= 256 KiB, else an
  *                    eighth of the launch), 2 = always an eighth of the launch, 3 = always an
  *                    eighth of a block
- *   "simple"         1 (default) = use the short-prologue kernel when the shape allows it
- *                    (not every threads/unroll/flag combination is compiled in; kvm_migrate
- *                    reports KVM_EINVAL for one that is not)
- *   "nt_load"        1 = nontemporal loads, 0 = plain
- *   "nt_store"       1 = nontemporal stores, 0 = plain
+ *   "sort_pairs"     order in which a migrate call's (context block, decoding block) pairs reach
+ *                    the kernel; the copy does not depend on it, the memory system does.
+ *                    1 (default) = by context block when the call names at least a quarter of
+ *                    the context pool (then most of the pool is read front to back: +4 % on
+ *                    calls of 800 of 1024 blocks whose rows are half read), else the caller's
+ *                    order; 0 = always the caller's order; 2 = always by context block
  *   "swap_mode"      3 (default) = chosen per call: mode 1, unless the copies of the call average
  *                        "swap_kernel_below" bytes or more each or the pinned pools are not mapped
  *                        for device access, then mode 2,
  *                    1 = copy kernel that reads/writes the pinned pools in place: one launch
- *                        per 432 blocks whatever their size, about 0.1 ms of host time for 2048
+ *                        per 864 blocks whatever their size, about 0.1 ms of host time for 2048
  *                        blocks, 97-100 % of the link,
  *                    2 = hipMemcpyAsync per run of blocks consecutive on both sides, K pool on
  *                        the caller's stream and V pool on a second stream forked from and
  *                        joined back into it: two runtime calls per block (4-5 ms of host time
  *                        for 2048 blocks), 97-98 % of the link for copies of 4 MiB, less below,
  *                    0 = the same with both pools on the caller's stream (87 %)
- *   "swap_wgs"       workgroups per pool kind of the swap kernel for a swap-out, 1..4096.  Default 8:
- *                    99 % of the link on an idle GPU and 96 % while other kernels saturate HBM
- *   "swap_wgs_in"    the same for a swap-in.  Default 10: 98 % idle, 98 % beside kernels that
- *                    saturate HBM, where 8 workgroups fall to 86 %; more workgroups slow the
- *                    kernels beside the swap (12: +5 %, 16: +20 %, 32: several times)
+ *   "swap_wgs"       workgroups per pool kind of the swap kernel for a swap-out, 1..4096; a
+ *                    workgroup keeps 4 KiB in flight.  Default 16: 99 % of the link on an idle GPU,
+ *                    97 % while other kernels saturate HBM, and a migration beside it 2-3 % slower
+ *   "swap_wgs_in"    the same for a swap-in.  Default 16: 99 % idle, 85 % beside kernels that
+ *                    saturate HBM, a migration beside it 2-3 % slower; with a swap-out and a swap-in
+ *                    in flight together, 46 GB/s each way (two large copies both ways: 49-52 down,
+ *                    30-57 up).  The trade is between the swap's share of the link while HBM is
+ *                    saturated and what the kernels beside it lose: 18 workgroups 94 % and 3.5 %,
+ *                    20: 96 % and 4 %, 36: 98 % and 15 %, 64 and more: several times slower
  *   "swap_kernel_below"  bytes per copy under which mode 3 takes the kernel (default 4 GiB, i.e.
  *                    always; 2 MiB hands large slabs to the copy engines)
+ * A library built with -DKVM_EXPLORE (sweeps and the tests that show every kernel flavour
+ * copies the same bytes; never shipped) knows more names: the workgroup shape, cache
+ * policy and tile size of the copy kernel.
  * kvm_get_option returns the value or KVM_EINVAL (as int64) for an unknown name.
  */
 int kvm_set_option(const char *name, int64_t value);
@@ -208,24 +220,30 @@ int64_t kvm_get_option(const char *name);
  * out[4] = kernel launches, out[5] = payload bytes per block (K+V, this rank's share),
  * out[6] = 1 when the short-prologue kernel (kvm_copy_simple_kernel) serves the shape,
  * out[7] = work-items (workgroups x workgroup size) of the largest launch, which the
- * library keeps below 2^32 by splitting the block list over more launches.
+ * library keeps below 2^32 by splitting the block list over more launches,
+ * out[8] = 16-byte vectors each lane moves, out[9] = index pairs one launch carries at most
+ * (864 when the context pools and a destination pool of dst_num_blocks blocks all have at
+ * most 65536 blocks, so that a pair packs into 32 bits; else 432; fewer for huge blocks).
+ * dst_num_blocks <= 0 = unknown (plans for 432).
  * Needs the sources registered (alignment of their bases picks the vector width), except
- * with dst_k == dst_v == NULL: then the plan is pure arithmetic, touches no device, and
- * takes every pool for 16-byte aligned.
+ * with dst_k == dst_v == NULL: then the plan is pure arithmetic, touches no device, takes
+ * every pool for 16-byte aligned and the context pools for dst_num_blocks blocks each.
  */
 int kvm_migrate_plan(const KvmGeom *geom, int64_t n, const void *dst_k, const void *dst_v,
-                     int64_t out[8]);
+                     int64_t dst_num_blocks, int64_t out[10]);
 
 /*
  * How kvm_swap would serve these lists at this slab size under the current options, for
  * tests and reports (no counterpart in the reference): out[0] = implementation taken (0, 1
  * or 2, as "swap_mode" numbers them), out[1] = copies per pool = runs of blocks consecutive
  * on both sides, out[2] = kernel launches (mode 1, else 0), out[3] = workgroups per pool
- * kind of each launch (mode 1, else 0; swap-in and swap-out have their own counts).  Touches
+ * kind of each launch (mode 1, else 0; swap-in and swap-out have their own counts).
+ * n_gpu_blocks / n_host_blocks: the pools' sizes, which decide how many blocks one launch
+ * carries (864 when both are at most 65536, else 432; <= 0 = unknown, plans for 432).  Touches
  * no device and no pool (so it cannot see whether pinned pools are mapped for the kernel).
  */
 int kvm_swap_plan(const int64_t *src_ids, const int64_t *dst_ids, int64_t n, int64_t slab_bytes,
-                  int is_swap_in, int64_t out[4]);
+                  int is_swap_in, int64_t n_gpu_blocks, int64_t n_host_blocks, int64_t out[4]);
 
 /*
  * Test hook (no counterpart in the reference): n / d computed the way the kernel computes

@@ -31,6 +31,18 @@ def kvm():
     return cabi
 
 
+@pytest.fixture(scope="session")
+def kvm_explore():
+    """The same binding over the exploration build (-DKVM_EXPLORE: every kernel flavour and
+    the knobs that select them).  A library of its own: its registry and options are not the
+    product's."""
+    from distserve_amd import cabi
+
+    path = os.path.join(ROOT, "tests", "lib_explore", "libkvmove.so")
+    assert os.path.exists(path), "tests/lib_explore/libkvmove.so is not built: python distserve_amd/csrc/build.py"
+    return cabi.Binding(path)
+
+
 @pytest.fixture()
 def fresh_registry(kvm):
     kvm.reset()

@@ -19,16 +19,17 @@ def stream_handle() -> int:
     return torch.cuda.current_stream().cuda_stream
 
 
-def upload_and_register(g: oracle.Geom, src_k: List[List[torch.Tensor]], src_v: List[List[torch.Tensor]]):
-    """Copies every context rank's pools to the GPU and registers them; returns the GPU
-    tensors (the caller keeps them alive)."""
+def upload_and_register(g: oracle.Geom, src_k: List[List[torch.Tensor]], src_v: List[List[torch.Tensor]], kvm=cabi):
+    """Copies every context rank's pools to the GPU and registers them with `kvm` (the
+    product's binding unless another build's is given); returns the GPU tensors (the caller
+    keeps them alive)."""
     dev_k = [[t.cuda() for t in row] for row in src_k]
     dev_v = [[t.cuda() for t in row] for row in src_v]
     for p in range(g.ctx_pp):
         for t in range(g.ctx_tp):
             k, v = dev_k[p][t], dev_v[p][t]
-            cabi.register_source(g.ctx_pp, g.ctx_tp, p, t, g.num_layers, g.num_kv_heads,
-                                 k.data_ptr(), v.data_ptr(), k.numel() * k.element_size())
+            kvm.register_source(g.ctx_pp, g.ctx_tp, p, t, g.num_layers, g.num_kv_heads,
+                                k.data_ptr(), v.data_ptr(), k.numel() * k.element_size())
     return dev_k, dev_v
 
 
@@ -53,12 +54,12 @@ def guards_intact(whole: torch.Tensor) -> bool:
             and torch.equal(got[-GUARD:].view(torch.uint8), margin.view(torch.uint8)))
 
 
-def gpu_migrate(g: oracle.Geom, ci, di, nb_dst: int, dtype=torch.float16):
+def gpu_migrate(g: oracle.Geom, ci, di, nb_dst: int, dtype=torch.float16, kvm=cabi):
     """Runs kvm_migrate into canary-filled destination pools; returns them on the CPU.  The
     pools have canary margins on both sides, which must survive."""
     dst_k, whole_k = guarded_canary_pool(g.dec_pool_shape(nb_dst), dtype)
     dst_v, whole_v = guarded_canary_pool(g.dec_pool_shape(nb_dst), dtype)
-    cabi.migrate(kvm_geom(g), ci, di, dst_k.data_ptr(), dst_v.data_ptr(), nb_dst, stream_handle())
+    kvm.migrate(kvm_geom(g), ci, di, dst_k.data_ptr(), dst_v.data_ptr(), nb_dst, stream_handle())
     torch.cuda.synchronize()
     assert guards_intact(whole_k) and guards_intact(whole_v), "a write strayed outside the destination pool"
     return dst_k.cpu(), dst_v.cpu()

@@ -18,7 +18,7 @@
 // with the geometry in template constants.  Launches rotate over windows of the buffers, or
 // draw fresh block lists, so that no launch finds its bytes in the 256 MB last-level cache.
 //
-// Build: hipcc --offload-arch=gfx950 -O3 hbm_probe.hip -o hbm_probe (distserve_amd/csrc/build.py does it).
+// Build: make -C tests/hbm_probe (hipcc --offload-arch=gfx950 -O3 hbm_probe.hip -o hbm_probe).
 
 #include <hip/hip_runtime.h>
 

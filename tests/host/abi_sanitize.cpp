@@ -35,12 +35,11 @@ static KvmGeom geom(int64_t L, int64_t H, int64_t B, int64_t D, int64_t s, int c
 
 int main()
 {
-    EXPECT(kvm_version() >= 100);
+    EXPECT(kvm_version() / 10000 == KVM_ABI_MAJOR);
     EXPECT(std::strlen(kvm_last_error()) == 0);
 
     // options: every name, valid and invalid values, unknown and null names
-    const char *names[] = {"tile_bytes", "threads", "unroll", "nt_load", "nt_store", "swap_mode", "swap_wgs", "swap_wgs_in",
-                           "lds_pad", "wave_contig", "xcd_map", "simple"};
+    const char *names[] = {"swap_mode", "swap_wgs", "swap_wgs_in", "swap_kernel_below", "xcd_map", "sort_pairs"};
     for (const char *n : names) {
         const int64_t old = kvm_get_option(n);
         EXPECT(kvm_set_option(n, old) == KVM_OK);
@@ -48,6 +47,7 @@ int main()
         EXPECT(kvm_get_option(n) == old);
     }
     EXPECT(kvm_set_option("no_such_option", 1) == KVM_EINVAL);
+    EXPECT(kvm_set_option("threads", 64) == KVM_EINVAL);        // a knob of the exploration build only
     EXPECT(kvm_set_option(nullptr, 1) == KVM_EINVAL);
     EXPECT(kvm_get_option(nullptr) == KVM_EINVAL);
     EXPECT(std::strlen(kvm_last_error()) > 0);
@@ -74,29 +74,39 @@ int main()
     EXPECT(kvm_migrate(&bad, ci.data(), di.data(), 1, fake_k, fake_v, 8, nullptr) == KVM_EINVAL);
     bad = geom(1 << 20, 1 << 10, 16, 128, 2);                   // a block beyond 4 GiB
     EXPECT(kvm_migrate(&bad, ci.data(), di.data(), 1, fake_k, fake_v, 8, nullptr) == KVM_EINVAL);
-    int64_t plan[8];
-    EXPECT(kvm_migrate_plan(&g, 10, fake_k, fake_v, nullptr) == KVM_EINVAL);
-    EXPECT(kvm_migrate_plan(&g, 10, fake_k, fake_v, plan) == KVM_ENOTREG);
+    int64_t plan[10];
+    EXPECT(kvm_migrate_plan(&g, 10, fake_k, fake_v, 64, nullptr) == KVM_EINVAL);
+    EXPECT(kvm_migrate_plan(&g, 10, fake_k, fake_v, 64, plan) == KVM_ENOTREG);
     KvmGeom other = g;
     other.ctx_instance = 3;                                     // no instance has anything registered
-    EXPECT(kvm_migrate_plan(&other, 10, fake_k, fake_v, plan) == KVM_ENOTREG);
+    EXPECT(kvm_migrate_plan(&other, 10, fake_k, fake_v, 64, plan) == KVM_ENOTREG);
 
     // Launch sizes, as pure arithmetic (null pools: nothing registered, no device touched).
     // A launch is 2 * tiles * blocks workgroups of 64 lanes and must stay below 2^32 work-items,
     // so big blocks get fewer index pairs per launch instead of a launch the runtime refuses.
-    EXPECT(kvm_migrate_plan(&g, -1, nullptr, nullptr, plan) == KVM_EINVAL);
+    EXPECT(kvm_migrate_plan(&g, -1, nullptr, nullptr, 0, plan) == KVM_EINVAL);
     {
-        // LLaMA-2-7B 1 -> 1: 4 MiB per pool kind per block = 4096 tiles, 432 blocks per launch
+        // LLaMA-2-7B 1 -> 1: 4 MiB per pool kind per block = 4096 tiles; 432 blocks per launch out of
+        // pools of unknown size, 864 when every pool has at most 65536 blocks
         KvmGeom g7 = geom(32, 32, 16, 128, 2);
-        EXPECT(kvm_migrate_plan(&g7, 909, nullptr, nullptr, plan) == KVM_OK);
+        EXPECT(kvm_migrate_plan(&g7, 909, nullptr, nullptr, 0, plan) == KVM_OK);
         EXPECT(plan[0] == 8192 && plan[1] == 64 && plan[2] == 16 && plan[3] == 1 && plan[4] == 3 && plan[6] == 1);
         EXPECT(plan[5] == 8388608);
-        EXPECT(plan[7] == 2ll * 4096 * 432 * 64);
+        EXPECT(plan[7] == 2ll * 4096 * 432 * 64 && plan[8] == 1 && plan[9] == 432);
+        EXPECT(kvm_migrate_plan(&g7, 909, nullptr, nullptr, 4096, plan) == KVM_OK);
+        EXPECT(plan[4] == 2 && plan[7] == 2ll * 4096 * 864 * 64 && plan[9] == 864);
+        EXPECT(kvm_migrate_plan(&g7, 909, nullptr, nullptr, 65537, plan) == KVM_OK && plan[9] == 432);
+        // pp4 x tp4 context ranks feed one decoding rank: 16 segments = 2 groups of 8, and 900 pairs are
+        // 2 launches per group of 864 packed pairs (3 of 432 wide ones)
+        KvmGeom g16 = geom(8, 8, 16, 8, 2, 4, 4);
+        EXPECT(kvm_migrate_plan(&g16, 900, nullptr, nullptr, 1024, plan) == KVM_OK);
+        EXPECT(plan[3] == 16 && plan[4] == 4 && plan[6] == 0);
+        EXPECT(kvm_migrate_plan(&g16, 900, nullptr, nullptr, 0, plan) == KVM_OK && plan[4] == 6);
         // a 1 GiB block per pool kind (L 128 x H 128 x B 256 x D 128 x 2 bytes): 2^20 tiles, so at
         // most 31 blocks fit a launch (2 * 31 * 2^20 * 64 < 2^32 <= 2 * 32 * 2^20 * 64)
         KvmGeom big = geom(128, 128, 256, 128, 2);
         for (int64_t n : {1, 31, 32, 100, 432, 1000}) {
-            EXPECT(kvm_migrate_plan(&big, n, nullptr, nullptr, plan) == KVM_OK);
+            EXPECT(kvm_migrate_plan(&big, n, nullptr, nullptr, 4096, plan) == KVM_OK);
             EXPECT(plan[5] == 2ll << 30);
             EXPECT(plan[7] > 0 && plan[7] < (1ll << 32));
             EXPECT(plan[4] == (n + 30) / 31);
@@ -104,17 +114,14 @@ int main()
         }
         // the same through two context ranks whose head split does not nest (general kernel, 2 segments)
         KvmGeom big2 = geom(128, 128, 256, 128, 2, 1, 2);
-        EXPECT(kvm_migrate_plan(&big2, 100, nullptr, nullptr, plan) == KVM_OK);
+        EXPECT(kvm_migrate_plan(&big2, 100, nullptr, nullptr, 4096, plan) == KVM_OK);
         EXPECT(plan[3] == 2 && plan[6] == 0 && plan[7] < (1ll << 32) && plan[4] == 4);
-        // larger workgroups leave room for fewer tiles per launch
-        EXPECT(kvm_set_option("threads", 1024) == KVM_OK && kvm_set_option("unroll", 4) == KVM_OK);
-        EXPECT(kvm_migrate_plan(&big, 1000, nullptr, nullptr, plan) == KVM_OK);
-        EXPECT(plan[1] == 1024 && plan[7] < (1ll << 32));
-        EXPECT(kvm_set_option("threads", 64) == KVM_OK && kvm_set_option("unroll", 1) == KVM_OK);
-        // many small blocks: every launch of 432 pairs is far below the limit
+        // many small blocks: every launch of 432 (or 864) pairs is far below the limit
         KvmGeom small = geom(2, 2, 16, 8, 2);
-        EXPECT(kvm_migrate_plan(&small, 100000, nullptr, nullptr, plan) == KVM_OK);
+        EXPECT(kvm_migrate_plan(&small, 100000, nullptr, nullptr, 100000, plan) == KVM_OK);
         EXPECT(plan[4] == (100000 + 431) / 432 && plan[7] < (1ll << 32));
+        EXPECT(kvm_migrate_plan(&small, 60000, nullptr, nullptr, 65536, plan) == KVM_OK);
+        EXPECT(plan[4] == (60000 + 863) / 864 && plan[7] < (1ll << 32));
     }
 
     // handles and registration
@@ -128,7 +135,7 @@ int main()
     EXPECT(kvm_register_mem_handle(nullptr, h, 4, 4, pc, pc, 0) == KVM_EINVAL);
     EXPECT(kvm_register_mem_handle(h, h, 4, 4, nullptr, pc, 0) == KVM_EINVAL);
     EXPECT(kvm_register_mem_handle(h, h, 4, 4, pc, bad_pc, 0) == KVM_EINVAL);
-    h[0] = 0x4b564d4f56453033LL; h[1] = 1; h[2] = 0; h[3] = 4096; h[4] = 64;   // plausible but forged: checksum missing
+    h[0] = 0x4b564d4f56453034LL; h[1] = 1; h[2] = 0; h[3] = 4096; h[4] = 64;   // plausible but forged: checksum missing
     EXPECT(kvm_register_mem_handle(h, h, 4, 4, pc, pc, 0) == KVM_EHANDLE);
     EXPECT(std::strstr(kvm_last_error(), "not a kvmove memory handle") != nullptr);
     // well-formed handles of another process (pid 1), with the checksum word as the library computes it
@@ -182,13 +189,13 @@ int main()
 
     // the swap plan touches no device: run lists of many shapes through it
     int64_t sp[4];
-    EXPECT(kvm_swap_plan(ci.data(), di.data(), 1, 64, 0, nullptr) == KVM_EINVAL);
-    EXPECT(kvm_swap_plan(nullptr, di.data(), 1, 64, 0, sp) == KVM_EINVAL);
-    EXPECT(kvm_swap_plan(ci.data(), di.data(), 1, 0, 0, sp) == KVM_EINVAL);
-    EXPECT(kvm_swap_plan(nullptr, nullptr, 0, 64, 0, sp) == KVM_OK && sp[1] == 0);
+    EXPECT(kvm_swap_plan(ci.data(), di.data(), 1, 64, 0, 0, 0, nullptr) == KVM_EINVAL);
+    EXPECT(kvm_swap_plan(nullptr, di.data(), 1, 64, 0, 0, 0, sp) == KVM_EINVAL);
+    EXPECT(kvm_swap_plan(ci.data(), di.data(), 1, 0, 0, 0, 0, sp) == KVM_EINVAL);
+    EXPECT(kvm_swap_plan(nullptr, nullptr, 0, 64, 0, 0, 0, sp) == KVM_OK && sp[1] == 0);
     // the default takes the copy kernel whatever the slab size, with its own workgroup count per direction
-    EXPECT(kvm_swap_plan(ci.data(), di.data(), 5, 4 << 20, 0, sp) == KVM_OK && sp[0] == 1 && sp[3] == kvm_get_option("swap_wgs"));
-    EXPECT(kvm_swap_plan(ci.data(), di.data(), 5, 4 << 20, 1, sp) == KVM_OK && sp[0] == 1 && sp[3] == kvm_get_option("swap_wgs_in"));
+    EXPECT(kvm_swap_plan(ci.data(), di.data(), 5, 4 << 20, 0, 0, 0, sp) == KVM_OK && sp[0] == 1 && sp[3] == kvm_get_option("swap_wgs"));
+    EXPECT(kvm_swap_plan(ci.data(), di.data(), 5, 4 << 20, 1, 0, 0, sp) == KVM_OK && sp[0] == 1 && sp[3] == kvm_get_option("swap_wgs_in"));
     // with a threshold, large copies go to the copy engines as before
     EXPECT(kvm_set_option("swap_kernel_below", 2 << 20) == KVM_OK);
     for (int round = 0; round < 200; ++round) {
@@ -202,11 +209,15 @@ int main()
             if (i > 0 && !(a[(size_t)i] == a[(size_t)i - 1] + 1 && b[(size_t)i] == b[(size_t)i - 1] + 1)) ++runs;
         }
         const int64_t slab = (int64_t)1 << (rng() % 24);
-        EXPECT(kvm_swap_plan(a.data(), b.data(), n, slab, round & 1, sp) == KVM_OK);
+        // pools of 100000 blocks (ids up to there) need wide pairs; every third round plans for small pools
+        const bool small_pools = round % 3 == 0;
+        EXPECT(kvm_swap_plan(a.data(), b.data(), n, slab, round & 1, small_pools ? 65536 : 200000,
+                             small_pools ? 4096 : 200000, sp) == KVM_OK);
         EXPECT(sp[1] == runs);
         const int64_t want = runs > 0 && n * slab / runs < (2 << 20) ? 1 : 2;
         EXPECT(sp[0] == want);
-        EXPECT(sp[2] == (want == 1 ? (n + 431) / 432 : 0));
+        const int64_t per = small_pools ? 864 : 432;
+        EXPECT(sp[2] == (want == 1 ? (n + per - 1) / per : 0));
         if (failures) break;
     }
     EXPECT(kvm_set_option("swap_kernel_below", 1ll << 32) == KVM_OK);

@@ -23,18 +23,39 @@ def test_every_declared_symbol_is_exported(kvm):
         assert getattr(raw, name) is not None
 
 
-def test_version_and_options(kvm):
-    assert kvm.version() >= 100
-    assert kvm.get_option("tile_bytes") == 0 and kvm.get_option("threads") == 64 and kvm.get_option("unroll") == 1
-    old = kvm.get_option("unroll")
-    kvm.set_option("unroll", 8)
-    assert kvm.get_option("unroll") == 8
-    kvm.set_option("unroll", old)
-    for name, bad in (("tile_bytes", 5000), ("threads", 100), ("unroll", 3), ("nt_store", 2), ("swap_mode", 4),
-                      ("swap_wgs", 0), ("swap_wgs_in", 5000), ("swap_kernel_below", -1), ("nope", 1)):
+def test_version_and_options(kvm, kvm_explore):
+    header = open(os.path.join(ROOT, "include", "kvmove.h")).read()
+    major = int(re.search(r"#define KVM_ABI_MAJOR (\d+)", header).group(1))
+    words = int(re.search(r"#define KVM_HANDLE_WORDS (\d+)", header).group(1))
+    assert kvm.version() // 10000 == major and kvm.KVM_HANDLE_WORDS == words
+    assert kvm.get_option("xcd_map") == 1 and kvm.get_option("sort_pairs") == 1
+    old = kvm.get_option("swap_wgs")
+    kvm.set_option("swap_wgs", 12)
+    assert kvm.get_option("swap_wgs") == 12
+    kvm.set_option("swap_wgs", old)
+    for name, bad in (("swap_mode", 4), ("swap_wgs", 0), ("swap_wgs_in", 5000), ("swap_kernel_below", -1),
+                      ("xcd_map", 4), ("sort_pairs", 3), ("nope", 1)):
         with pytest.raises(kvm.KvmError) as e:
             kvm.set_option(name, bad)
         assert e.value.code == kvm.KVM_EINVAL
+    # the product carries one kernel flavour and none of the knobs that select others ...
+    for name in ("tile_bytes", "threads", "unroll", "nt_load", "nt_store", "wave_contig", "lds_pad", "simple"):
+        with pytest.raises(kvm.KvmError):
+            kvm.get_option(name)
+        with pytest.raises(kvm.KvmError):
+            kvm.set_option(name, 0)
+    # ... the exploration build has them, with the product's flavour as the default
+    x = kvm_explore
+    assert x.version() == kvm.version()
+    assert x.get_option("tile_bytes") == 0 and x.get_option("threads") == 64 and x.get_option("unroll") == 1
+    assert x.get_option("nt_load") == 1 and x.get_option("nt_store") == 1 and x.get_option("simple") == 1
+    x.set_option("unroll", 8)
+    assert x.get_option("unroll") == 8
+    x.set_option("unroll", 1)
+    for name, bad in (("tile_bytes", 5000), ("threads", 100), ("unroll", 3), ("nt_store", 2), ("max_pairs", 865)):
+        with pytest.raises(x.KvmError) as e:
+            x.set_option(name, bad)
+        assert e.value.code == x.KVM_EINVAL
 
 
 def test_swap_plan_takes_the_kernel_by_default_and_the_engines_above_a_threshold(kvm):
@@ -42,12 +63,18 @@ def test_swap_plan_takes_the_kernel_by_default_and_the_engines_above_a_threshold
     direction.  With a "swap_kernel_below" threshold, calls whose copies average that many
     bytes go to the copy engines; runs of blocks consecutive on both sides count as one copy."""
     assert kvm.get_option("swap_mode") == 3 and kvm.get_option("swap_kernel_below") == 1 << 32
-    assert kvm.get_option("swap_wgs") == 8 and kvm.get_option("swap_wgs_in") == 10
+    assert kvm.get_option("swap_wgs") == 16 and kvm.get_option("swap_wgs_in") == 16
     scattered = ([5, 9, 2, 7], [1, 8, 3, 6])
     assert kvm.swap_plan(*scattered, 4 << 20) == {"mode": 1, "copies_per_pool": 4, "launches": 1,
-                                                  "workgroups_per_pool_kind": 8}
-    assert kvm.swap_plan(*scattered, 4 << 20, is_swap_in=True)["workgroups_per_pool_kind"] == 10
-    assert kvm.swap_plan(list(range(0, 2000, 2)), list(range(1000)), 4096)["launches"] == 3   # 432 blocks per launch
+                                                  "workgroups_per_pool_kind": 16}
+    kvm.set_option("swap_wgs_in", 18)
+    assert kvm.swap_plan(*scattered, 4 << 20, is_swap_in=True)["workgroups_per_pool_kind"] == 18
+    kvm.set_option("swap_wgs_in", 16)
+    # pools of unknown size: 432 blocks per launch; pools of at most 65536 blocks: 864
+    ids = (list(range(0, 2000, 2)), list(range(1000)))
+    assert kvm.swap_plan(*ids, 4096)["launches"] == 3
+    assert kvm.swap_plan(*ids, 4096, n_gpu_blocks=4096, n_host_blocks=65536)["launches"] == 2
+    assert kvm.swap_plan(*ids, 4096, n_gpu_blocks=4096, n_host_blocks=65537)["launches"] == 3
     assert kvm.swap_plan([], [], 4096) == {"mode": 2, "copies_per_pool": 0, "launches": 0, "workgroups_per_pool_kind": 0}
     kvm.set_option("swap_kernel_below", 2 << 20)
     try:
@@ -103,29 +130,34 @@ def test_argument_errors_need_no_gpu(kvm, fresh_registry):
     assert e.value.code == kvm.KVM_EINVAL
 
 
-def test_launches_stay_below_the_grid_limit_for_blocks_of_any_size(kvm, fresh_registry):
+def test_launches_stay_below_the_grid_limit_for_blocks_of_any_size(kvm, kvm_explore, fresh_registry):
     """A launch is 2 x tiles x blocks workgroups of `threads` lanes; the runtime refuses 2^32
     work-items and more, so the block list is split over more launches before anything is
     enqueued.  Pure arithmetic: null pools, nothing registered, no device."""
-    plan = kvm.migrate_plan(kvm.geom(32, 32, 16, 128, 2), 909, 0, 0)          # LLaMA-2-7B, 1 -> 1
+    plan = kvm.migrate_plan(kvm.geom(32, 32, 16, 128, 2), 909, 0, 0)          # LLaMA-2-7B, 1 -> 1, pools of any size
     assert plan["launches"] == 3 and plan["simple_kernel"] == 1 and plan["max_work_items"] == 2 * 4096 * 432 * 64
+    assert plan["pairs_per_launch"] == 432 and plan["threads"] == 64 and plan["vectors_per_lane"] == 1
+    plan = kvm.migrate_plan(kvm.geom(32, 32, 16, 128, 2), 909, 0, 0, 4096)    # ... pools of 4096 blocks: packed pairs
+    assert plan["launches"] == 2 and plan["pairs_per_launch"] == 864 and plan["max_work_items"] == 2 * 4096 * 864 * 64
+    assert kvm.migrate_plan(kvm.geom(32, 32, 16, 128, 2), 909, 0, 0, 65537)["pairs_per_launch"] == 432
     big = kvm.geom(128, 128, 256, 128, 2)                                      # 1 GiB per pool kind per block
     tiles = (1 << 30) // 1024
     for n in (1, 31, 32, 433, 5000):
-        plan = kvm.migrate_plan(big, n, 0, 0)
+        plan = kvm.migrate_plan(big, n, 0, 0, 4096)
         per_launch = (2**32 - 1) // (2 * 64) // tiles                          # 31, short of the padding allowance
         assert plan["payload_bytes_per_block"] == 2 << 30
         assert plan["launches"] == -(-n // per_launch)
         assert 0 < plan["max_work_items"] < 2**32
     for threads, unroll in ((256, 4), (1024, 4)):
-        kvm.set_option("threads", threads)
-        kvm.set_option("unroll", unroll)
+        kvm_explore.set_option("threads", threads)
+        kvm_explore.set_option("unroll", unroll)
         try:
-            plan = kvm.migrate_plan(big, 5000, 0, 0)
-            assert plan["threads"] == threads and 0 < plan["max_work_items"] < 2**32
+            plan = kvm_explore.migrate_plan(big, 5000, 0, 0, 4096)
+            assert plan["threads"] == threads and plan["vectors_per_lane"] == unroll
+            assert 0 < plan["max_work_items"] < 2**32
         finally:
-            kvm.set_option("threads", 64)
-            kvm.set_option("unroll", 1)
+            kvm_explore.set_option("threads", 64)
+            kvm_explore.set_option("unroll", 1)
     # with real (non-null) destination pointers the plan wants the sources registered, as before
     with pytest.raises(kvm.KvmError) as e:
         kvm.migrate_plan(big, 4, 4096, 8192)
@@ -174,8 +206,8 @@ def test_row_of_a_tile_is_computed_without_a_divider_exactly(kvm):
         probes += [rng.randrange(0, 2**32) for _ in range(40)]
         for n in probes:
             if 0 <= n < 2**32:
-                assert kvm.lib.kvm_debug_divide(n, d) == n // d, (n, d)
-    assert kvm.lib.kvm_debug_divide(5, 0) == 2**32 - 1
+                assert kvm.debug_divide(n, d) == n // d, (n, d)
+    assert kvm.debug_divide(5, 0) == 2**32 - 1
 
 
 def test_the_package_refuses_to_import_without_its_libraries(tmp_path):
@@ -209,14 +241,12 @@ def test_the_alternate_namespace_build_registers_the_same_schemas_beside_the_fir
 
 
 def test_the_ceiling_probe_is_built_and_explains_its_flags():
-    """The stand-alone probe of the memory system's ceilings is built beside the libraries
-    (no GPU call happens before its arguments are read)."""
+    """The stand-alone probe of the memory system's ceilings (a fixture of the bench-target
+    test) is built (no GPU call happens before its arguments are read)."""
     import subprocess
 
-    import distserve_amd
-
-    probe = os.path.join(os.path.dirname(distserve_amd.TORCH_LIB_PATH), "hbm_probe")
-    assert os.path.exists(probe), "python distserve_amd/csrc/build.py builds it"
+    probe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "hbm_probe", "hbm_probe")
+    assert os.path.exists(probe), "make -C tests/hbm_probe builds it"
     run = subprocess.run([probe, "--no-such-flag"], capture_output=True, text=True)
     assert run.returncode == 2
     assert "--section" in run.stderr and "--quick" in run.stderr

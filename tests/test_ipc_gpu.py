@@ -87,10 +87,10 @@ SPEC = {"layers": 8, "kv_heads": 8, "head_dim": 64, "tp": 2, "pp": 2, "blocks": 
 
 
 def sealed(words) -> int:
-    """The check word of a handle, as the library computes it over the 16 words before it."""
+    """The check word of a handle, as the library computes it over the 17 words before it."""
     mask = (1 << 64) - 1
     x = 0x5A5A5A5A5A5A5A5A
-    for w in words[:16]:
+    for w in words[:17]:
         x = (((x << 7) | (x >> 57)) & mask) ^ (w & mask)
     return x - (1 << 64) if x >> 63 else x
 
@@ -181,13 +181,38 @@ def test_context_instance_in_another_process_tp2pp2_to_tp4_every_rank_against_or
         lie = list(handles[0][0][0])
         lie[6] *= 64                                    # the allocation's size, as the exporter tells it
         lie[4] = lie[6] - (lie[3] - lie[5])             # a pool that runs to the claimed end
-        lie[16] = sealed(lie)
+        lie[17] = sealed(lie)
         with pytest.raises(kvm.KvmError) as e:
             kvm.register_mem_handle(lie, lie, 8, 8, [1, 0, 1, 0], [1, 0, 1, 0])
         assert e.value.code == kvm.KVM_EHANDLE and "the mapping holds" in str(e.value)
         assert kvm.opened_handles() == 0
+        # a registration whose V handle fails after its K handle has been mapped leaves nothing mapped
+        k00, v00 = handles[0][0]
+        broken = list(v00)
+        broken[4] = 0                                   # names no memory
+        broken[17] = sealed(broken)
+        with pytest.raises(kvm.KvmError) as e:
+            kvm.register_mem_handle(k00, broken, 8, 8, [2, 0, 2, 0], [1, 0, 1, 0])
+        assert e.value.code == kvm.KVM_EHANDLE and "names no memory" in str(e.value)
+        assert kvm.opened_handles() == 0
+        # handles whose exporter had no allocation id to give (the id bits cleared here): the rank's K
+        # and V pools still share the mapping their registration call opens, and a second
+        # registration maps the allocation anew instead of trusting the old mapping
+        anonymous = []
+        for h in (k00, v00):
+            h = list(h)
+            h[7] &= 0xFF
+            h[17] = sealed(h)
+            anonymous.append(h)
+        for _ in range(2):
+            kvm.register_mem_handle(*anonymous, 8, 8, [2, 0, 2, 0], [1, 0, 1, 0], ctx_instance=5)
+            assert kvm.opened_handles() == len({(h[1], h[5]) for h in anonymous})
+        kvm.reset()
+        assert kvm.opened_handles() == 0
         # ... and while the allocation is open under its true size, it unbinds nothing
         dec.register_kvcache_mem_handles(ctx_config, handles)
+        # a pool that is bound again elsewhere leaves its old mapping without a user: it is closed
+        # (here instance 5's binding went with the reset above; nothing but instance 0's is open)
         # one mapping per allocation of the other process, however many pools lie in it and
         # however often they are registered
         allocations = {(h[1], h[5]) for row in handles for pair in row for h in pair}
@@ -292,6 +317,33 @@ def test_context_and_decoding_instances_as_sibling_processes(kvm, tmp_path):
         ctx.close()
     assert ctx.proc.returncode == 0 and dec.proc.returncode == 0, (
         open(ctx.log_path).read()[-2000:] + open(dec.log_path).read()[-2000:])
+
+
+def test_a_handle_with_this_pid_but_another_nonce_is_not_taken_for_a_local_pointer(kvm):
+    """Two processes in different pid namespaces can share a pid.  A handle resolves to its raw
+    pointer only when pid AND the exporter's random word match this process; otherwise it goes
+    the way of every foreign handle (here the runtime refuses to map this process's own
+    export, or maps it: either way the pointer in the handle is not dereferenced as local)."""
+    kvm.reset()
+    g = oracle.Geom(2, 2, 16, 8, 2)
+    pool = torch.zeros(g.ctx_pool_shape(4), dtype=torch.float16, device="cuda")
+    nbytes = pool.numel() * 2
+    own = kvm.get_mem_handle(pool.data_ptr(), nbytes)
+    assert own[1] == os.getpid() and own[16] != 0
+    kvm.register_mem_handle(own, own, 2, 2, [1, 0, 1, 0], [1, 0, 1, 0])
+    assert kvm.opened_handles() == 0                           # its own: the pointer itself
+    kvm.reset()
+    other = list(own)
+    other[16] ^= 0x5555                                        # same pid, another process's random word
+    other[17] = sealed(other)
+    try:
+        kvm.register_mem_handle(other, other, 2, 2, [1, 0, 1, 0], [1, 0, 1, 0])
+    except kvm.KvmError as e:
+        assert e.code == kvm.KVM_EHANDLE and "could not be opened" in str(e)
+        assert kvm.opened_handles() == 0
+    else:
+        assert kvm.opened_handles() == 1                       # bound through a mapping, not through the raw pointer
+    kvm.reset()
 
 
 def test_own_handles_still_resolve_without_ipc_whatever_the_pool_size(kvm):

@@ -20,8 +20,8 @@ def check_case(kvm, g, nb_src, nb_dst, ci, di, seed=1, dtype=torch.float16):
     kvm.reset()
     src_k = make_src_pools(g, nb_src, seed, dtype)
     src_v = make_src_pools(g, nb_src, seed + 500, dtype)
-    keep = upload_and_register(g, src_k, src_v)
-    got_k, got_v = gpu_migrate(g, ci, di, nb_dst, dtype)
+    keep = upload_and_register(g, src_k, src_v, kvm)
+    got_k, got_v = gpu_migrate(g, ci, di, nb_dst, dtype, kvm)
     want_k, want_v = oracle_migrate(g, src_k, src_v, ci, di, nb_dst, dtype)
     assert same_bits(got_k, want_k), "K pool differs from the oracle"
     assert same_bits(got_v, want_v), "V pool differs from the oracle"
@@ -139,14 +139,77 @@ def test_misaligned_pool_bases_pick_a_narrower_vector(kvm):
     kvm.reset()
 
 
-@pytest.mark.parametrize("n", [0, 1, 431, 432, 433, 865, 1000])
+@pytest.mark.parametrize("n", [0, 1, 431, 432, 433, 863, 864, 865, 1000, 1729, 2000])
 def test_list_lengths_around_the_per_launch_limit(kvm, n):
-    """One launch carries 432 index pairs; longer lists split into several launches."""
+    """One launch carries 864 index pairs (pools of at most 65536 blocks: a pair packs into 32
+    bits); longer lists split into several launches."""
     g = oracle.Geom(2, 2, 16, 8, 2)
     gen = torch.Generator().manual_seed(n)
     ci = torch.randint(0, 64, (n,), generator=gen).tolist()          # context blocks may repeat
-    di = torch.randperm(1200, generator=gen)[:n].tolist()
-    check_case(kvm, g, 64, 1200, ci, di, seed=5)
+    di = torch.randperm(2100, generator=gen)[:n].tolist()
+    check_case(kvm, g, 64, 2100, ci, di, seed=5)
+
+
+@pytest.mark.parametrize("n", [1, 432, 433, 900])
+@pytest.mark.parametrize("big", ["destination", "source"])
+def test_pools_of_more_than_65536_blocks_take_wide_index_pairs(kvm, n, big):
+    """Block ids beyond 16 bits travel as two int32 (432 pairs per launch).  The blocks are
+    64 bytes here, so that 70000 of them are a small pool; the top ids are used."""
+    g = oracle.Geom(1, 1, 4, 4, 2)
+    nb_src, nb_dst = (64, 70000) if big == "destination" else (70000, 1200)
+    gen = torch.Generator().manual_seed(n)
+    ci = (torch.randint(0, nb_src, (n,), generator=gen)).tolist()
+    di = torch.randperm(nb_dst, generator=gen)[:n].tolist()
+    ci[0], di[0] = nb_src - 1, nb_dst - 1
+    kvm.reset()
+    keep = upload_and_register(g, make_src_pools(g, nb_src, 1), make_src_pools(g, nb_src, 2), kvm)
+    dst = canary_pool(g.dec_pool_shape(nb_dst)).cuda()
+    plan = kvm.migrate_plan(kvm_geom(g), n, dst.data_ptr(), dst.data_ptr(), nb_dst)
+    assert plan["pairs_per_launch"] == 432 and plan["launches"] == -(-n // 432)
+    del keep, dst
+    check_case(kvm, g, nb_src, nb_dst, ci, di, seed=9)
+
+
+@pytest.mark.parametrize("order", ["scattered", "neighbours", "descending"])
+def test_many_segments_times_many_pairs_split_into_launches_both_ways(kvm, order):
+    """pp4 x tp4 context ranks feed one decoding rank (16 segments: two groups of 8) and the
+    list has 1800 pairs (three launches of 864 per group): the launch splitter's two loops
+    multiply, and a mostly-neighbouring list keeps its order over all six launches."""
+    g = oracle.Geom(8, 8, 4, 8, 2, 4, 4, 1, 1, 0, 0)
+    n, nb_src, nb_dst = 1800, 2000, 2200
+    gen = torch.Generator().manual_seed(3)
+    if order == "scattered":
+        ci = torch.randperm(nb_src, generator=gen)[:n].tolist()
+    elif order == "neighbours":
+        ci = list(range(7, 7 + 700)) + list(range(1200, 1200 + 600)) + list(range(800, 800 + 500))
+    else:
+        ci = list(range(nb_src - 1, nb_src - 1 - n, -1))
+    di = torch.randperm(nb_dst, generator=gen)[:n].tolist()
+    kvm.reset()
+    keep = upload_and_register(g, make_src_pools(g, nb_src, 1), make_src_pools(g, nb_src, 2), kvm)
+    dst = canary_pool(g.dec_pool_shape(nb_dst)).cuda()
+    plan = kvm.migrate_plan(kvm_geom(g), n, dst.data_ptr(), dst.data_ptr(), nb_dst)
+    assert plan["segments"] == 16 and plan["pairs_per_launch"] == 864 and plan["launches"] == 2 * 3
+    del keep, dst
+    check_case(kvm, g, nb_src, nb_dst, ci, di, seed=31)
+
+
+@pytest.mark.parametrize("sort_pairs", [0, 1, 2])
+@pytest.mark.parametrize("n,nb_src", [(40, 64), (200, 256), (200, 4000), (1000, 1100)])
+def test_the_order_of_the_pairs_is_the_librarys_to_choose(kvm, sort_pairs, n, nb_src):
+    """A call that names a quarter of the context pool or more has its pairs put in the order
+    of their context blocks before they reach the kernel ("sort_pairs" 1; 2 always, 0
+    never); the copy is the same whatever the order, repeated context blocks included."""
+    g = oracle.Geom(2, 4, 16, 32, 2, 1, 2, 1, 1)
+    gen = torch.Generator().manual_seed(n + nb_src)
+    ci = torch.randint(0, nb_src, (n,), generator=gen).tolist()      # with repeats
+    di = torch.randperm(n + 50, generator=gen)[:n].tolist()
+    old = kvm.get_option("sort_pairs")
+    kvm.set_option("sort_pairs", sort_pairs)
+    try:
+        check_case(kvm, g, nb_src, n + 50, ci, di, seed=13)
+    finally:
+        kvm.set_option("sort_pairs", old)
 
 
 def test_more_context_ranks_than_one_launch_holds(kvm):
@@ -156,7 +219,7 @@ def test_more_context_ranks_than_one_launch_holds(kvm):
     kvm.reset()
     keep = upload_and_register(g, make_src_pools(g, 7, 1), make_src_pools(g, 7, 2))
     dst = canary_pool(g.dec_pool_shape(9)).cuda()
-    plan = kvm.migrate_plan(kvm_geom(g), 3, dst.data_ptr(), dst.data_ptr())
+    plan = kvm.migrate_plan(kvm_geom(g), 3, dst.data_ptr(), dst.data_ptr(), 9)
     assert plan["segments"] == 16 and plan["launches"] == 2
     del keep
     kvm.reset()
@@ -168,7 +231,9 @@ def test_more_context_ranks_than_one_launch_holds(kvm):
     (0, 256, 4, ((1, 1, 0), (0, 0, 0))), (32768, 256, 4, ((1, 1, 0),)), (0, 256, 8, ((1, 1, 0), (1, 1, 1))),
     (8192, 512, 2, ((1, 1, 0),)), (1 << 20, 512, 8, ((1, 1, 0), (0, 0, 0))), (16384, 1024, 4, ((1, 1, 0),)),
     (1024, 64, 4, ((1, 1, 1),)), (2048, 64, 1, ((1, 1, 0),))])
-def test_every_tuning_choice_copies_the_same_bytes(kvm, tile_bytes, threads, unroll, flavours):
+def test_every_tuning_choice_copies_the_same_bytes(kvm_explore, tile_bytes, threads, unroll, flavours):
+    """Through the exploration build: the product carries the first flavour only."""
+    kvm = kvm_explore
     names = ("tile_bytes", "threads", "unroll", "nt_load", "nt_store", "wave_contig")
     saved = {k: kvm.get_option(k) for k in names}
     try:
@@ -188,19 +253,22 @@ def test_every_tuning_choice_copies_the_same_bytes(kvm, tile_bytes, threads, unr
             kvm.set_option(k, v)
 
 
-def test_a_flavour_that_was_not_built_is_refused(kvm):
+def test_a_flavour_that_was_not_built_is_refused(kvm_explore):
+    kvm = kvm_explore
     g = oracle.Geom(2, 2, 16, 8, 2)
     kvm.reset()
-    keep = upload_and_register(g, make_src_pools(g, 3, 1), make_src_pools(g, 3, 2))
+    keep = upload_and_register(g, make_src_pools(g, 3, 1), make_src_pools(g, 3, 2), kvm)
     dst = canary_pool(g.dec_pool_shape(3)).cuda()
     old = kvm.get_option("unroll")
     try:
+        kvm.set_option("nt_load", 0)            # plain loads with nontemporal stores: built for a few shapes only
         kvm.set_option("unroll", 16)
         with pytest.raises(kvm.KvmError) as e:
             kvm.migrate(kvm_geom(g), [0], [1], dst.data_ptr(), dst.data_ptr(), 3, stream_handle())
         assert e.value.code == kvm.KVM_EINVAL and "no kernel was built" in str(e.value)
     finally:
         kvm.set_option("unroll", old)
+        kvm.set_option("nt_load", 1)
     torch.cuda.synchronize()
     assert same_bits(dst.cpu(), canary_pool(g.dec_pool_shape(3)))
     del keep
@@ -462,14 +530,20 @@ def test_configs_3_and_4_full_size_properties(kvm, make):
     kvm.reset()
 
 
-@pytest.mark.parametrize("xcd_map,simple", [(0, 0), (0, 1), (1, 0), (1, 1), (2, 0), (2, 1), (3, 1)])
-def test_every_id_to_work_mapping_copies_the_same_bytes(kvm, xcd_map, simple):
+@pytest.mark.parametrize("xcd_map,simple", [(0, 0), (0, 1), (1, 0), (1, 1), (2, 0), (2, 1), (3, 1), (1, None), (2, None)])
+def test_every_id_to_work_mapping_copies_the_same_bytes(kvm, kvm_explore, xcd_map, simple):
     """Workgroup ids are dealt to XCDs in contiguous chunks; with padding ids when the work
-    does not divide by 8 (odd tile counts, odd block counts)."""
-    saved = {k: kvm.get_option(k) for k in ("xcd_map", "simple")}
+    does not divide by 8 (odd tile counts, odd block counts).  simple None: the product (which
+    always takes the short-prologue kernel where the shape allows); 0/1: the exploration build."""
+    if simple is None:
+        simple = 1
+    else:
+        kvm = kvm_explore
+    saved = {k: kvm.get_option(k) for k in ("xcd_map",) + (("simple",) if kvm is kvm_explore else ())}
     try:
         kvm.set_option("xcd_map", xcd_map)
-        kvm.set_option("simple", simple)
+        if "simple" in saved:
+            kvm.set_option("simple", simple)
         gen = torch.Generator().manual_seed(17)
         for g, nb_src, nb_dst, n in [
                 (oracle.Geom(2, 16, 16, 128, 2), 40, 48, 37),                   # 128 KiB blocks: 128 tiles
@@ -485,14 +559,45 @@ def test_every_id_to_work_mapping_copies_the_same_bytes(kvm, xcd_map, simple):
             kvm.set_option(k, v)
 
 
-def test_random_geometries_pools_lists_and_tunings(kvm):
+@pytest.mark.parametrize("build", ["product", "exploration"])
+def test_random_geometries_pools_lists_and_tunings(kvm, kvm_explore, build):
     """300 seeded draws of everything at once: layer/head counts and splits (nesting or not),
     block and head sizes down to one element, 1/2/4-byte elements, pool sizes, index lists
-    with repeated sources, and every compiled tuning choice."""
+    with repeated sources, and -- in the exploration build -- the kernel flavours, tile
+    sizes and table forms (the product has one flavour; its draws vary its own options)."""
     import random
 
+    if build == "product":
+        rng = random.Random(21)
+        saved = {k: kvm.get_option(k) for k in ("xcd_map", "sort_pairs")}
+        try:
+            for case in range(300):
+                L, H = rng.choice([1, 2, 3, 4, 6, 8, 12]), rng.choice([1, 2, 3, 4, 6, 8, 12])
+                div = lambda n: [d for d in range(1, n + 1) if n % d == 0]    # noqa: E731
+                cpp, dpp, ctp, dtp = rng.choice(div(L)), rng.choice(div(L)), rng.choice(div(H)), rng.choice(div(H))
+                B, D = rng.choice([1, 2, 3, 4, 8, 16, 32]), rng.choice([1, 2, 3, 5, 8, 16, 40, 64, 80, 128])
+                s = rng.choice([1, 2, 2, 2, 4])
+                g = oracle.Geom(L, H, B, D, s, cpp, ctp, dpp, dtp, rng.randrange(dpp), rng.randrange(dtp))
+                nb_src, nb_dst = rng.randint(1, 12), rng.randint(1, 12)
+                n = rng.randint(0, nb_dst)
+                ci, di = [rng.randrange(nb_src) for _ in range(n)], rng.sample(range(nb_dst), n)
+                chosen = dict(xcd_map=rng.randrange(4), sort_pairs=rng.randrange(3))
+                for k, v in chosen.items():
+                    kvm.set_option(k, v)
+                try:
+                    check_case(kvm, g, nb_src, nb_dst, ci, di, seed=case + 1,
+                               dtype={1: torch.uint8, 2: torch.float16, 4: torch.float32}[s])
+                except AssertionError as e:
+                    raise AssertionError(f"case {case}: {g} {chosen} ctx {ci} dec {di}: {e}") from None
+        finally:
+            for k, v in saved.items():
+                kvm.set_option(k, v)
+        return
+    kvm = kvm_explore
+
     rng = random.Random(20)
-    names = ("threads", "unroll", "nt_load", "nt_store", "wave_contig", "tile_bytes", "xcd_map", "simple")
+    names = ("threads", "unroll", "nt_load", "nt_store", "wave_contig", "tile_bytes", "xcd_map", "simple", "packed",
+             "sort_pairs")
     saved = {k: kvm.get_option(k) for k in names}
     flavours = [(64, 1, 1, 1, 0), (64, 2, 1, 1, 0), (128, 1, 1, 1, 0), (256, 1, 1, 1, 0), (256, 4, 1, 1, 0),
                 (256, 8, 1, 1, 0), (512, 2, 1, 1, 0), (512, 8, 1, 1, 0), (1024, 4, 1, 1, 0), (64, 1, 0, 0, 0),
@@ -517,7 +622,7 @@ def test_random_geometries_pools_lists_and_tunings(kvm):
             threads, unroll, nt_load, nt_store, wave_contig = rng.choice(flavours)
             chosen = dict(threads=threads, unroll=unroll, nt_load=nt_load, nt_store=nt_store, wave_contig=wave_contig,
                           tile_bytes=rng.choice([0, 0, 0, 1024, 4096, 16384, 65536]), xcd_map=rng.randrange(4),
-                          simple=rng.randrange(2))
+                          simple=rng.randrange(2), packed=rng.randrange(2), sort_pairs=rng.randrange(3))
             for k, v in chosen.items():
                 kvm.set_option(k, v)
             try:
