@@ -52,6 +52,9 @@ def parse_args():
                          "(bridge queue -> scheduler -> engine -> op), batch_migrations off or on; "
                          "ipc: configuration 2's shape with the context pools in ANOTHER process (memory handles "
                          "over a pipe, hipIpc mapping), against the same pools in this process")
+    ap.add_argument("--request-blocks", type=int, nargs="*", default=None, metavar="N",
+                    help="handoff*/scheduler* patterns: instead of a configuration, 48 requests of N blocks each at the "
+                         "LLaMA-2-7B shape, one record per N (what the hand-off costs by prompt length)")
     ap.add_argument("--ipc-child", action="store_true", help=argparse.SUPPRESS)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-verify", action="store_true")
@@ -216,10 +219,14 @@ def host_call_cost_us(cabi, geom, w, dst_k, dst_v, stream, calls=64):
     return round(costs[len(costs) // 2], 2), round(costs[0], 2)
 
 
-def bench_migrate(config: int, pattern: str, steps: int, warmup: int, verify_result: bool = True,
+def bench_migrate(config: int, patterns, steps: int, warmup: int, verify_result: bool = True,
                   calibrate_copy: bool = False, ctx_tp=None, fresh_pools=False):
-    """Times one migration workload; returns (record, workload).  Pools are made, timed and
-    freed inside."""
+    """Times one migration workload under every call pattern of `patterns` ("request", "batch"),
+    all on ONE set of pools (two patterns of a configuration are then compared on the same
+    memory); returns (records in the order of `patterns`, workload).  Pools are made, timed
+    and freed inside."""
+    import gc
+
     import torch
 
     from distserve_amd import cabi, workloads
@@ -244,107 +251,113 @@ def bench_migrate(config: int, pattern: str, steps: int, warmup: int, verify_res
             cabi.register_source(w.ctx_pp, w.ctx_tp, p, t, s.num_layers, s.num_kv_heads,
                                  src_k[p][t].data_ptr(), src_v[p][t].data_ptr(),
                                  src_k[p][t].numel() * s.dtype_bytes)
-    calls = [(cabi.index_array(ci), cabi.index_array(di)) for ci, di in make_calls(w, pattern)]
-    plan = cabi.migrate_plan(geom, max(len(c[0]) for c in calls), dst_k.data_ptr(), dst_v.data_ptr(), w.dst_blocks)
-    launches_per_step = 0
-    for ci, _ in calls:
-        launches_per_step += cabi.migrate_plan(geom, len(ci), dst_k.data_ptr(), dst_v.data_ptr(),
-                                               w.dst_blocks)["launches"]
-
-    def step():
-        for ci, di in calls:
-            cabi.migrate(geom, ci, di, dst_k.data_ptr(), dst_v.data_ptr(), w.dst_blocks, stream.cuda_stream)
-
-    for _ in range(warmup):
-        step()
-    # no collector pass inside the timed region (a full one over torch's modules takes 35 ms)
-    import gc
-
-    gc.collect()
-    gc.freeze()
-    torch.cuda.synchronize()
-    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    start.record(stream)
-    for _ in range(steps):
-        step()
-    stop.record(stream)
-    torch.cuda.synchronize()
-    elapsed_ms = start.elapsed_time(stop)
-    ms_per_step = elapsed_ms / steps
-
-    # a second pass with an event between steps, for the spread (median and best step)
-    marks = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
-    marks[0].record(stream)
-    for i in range(steps):
-        step()
-        marks[i + 1].record(stream)
-    torch.cuda.synchronize()
-    per_step_ms = sorted(marks[i].elapsed_time(marks[i + 1]) for i in range(steps))
-
     payload = w.payload_bytes                       # bytes the decoding rank receives per step
     hbm_bytes = 2 * payload                         # each byte read once and written once
-    hbm_gbps = hbm_bytes / (ms_per_step * 1e-3) / 1e9
-    launch_us = elapsed_ms * 1e3 / (steps * launches_per_step)
-    bytes_per_launch = hbm_bytes / launches_per_step
-
-    bit_exact = verify(w, src_k, src_v, dst_k, dst_v) if verify_result else None
-    host_call_us, host_call_us_min = host_call_cost_us(cabi, geom, w, dst_k, dst_v, stream)
-    copy_ceiling = time_plain_copy(cabi, stream) if calibrate_copy else None
-
-    tuning = {"threads": plan["threads"], "vectors_per_lane": plan["vectors_per_lane"],
-              "pairs_per_launch": plan["pairs_per_launch"],
-              **{k: cabi.get_option(k) for k in ("xcd_map", "sort_pairs")}}
-    # the name the kernel trace shows, shortened: vector type, lanes, vectors per lane, index-table form
-    kernel = (("kvm_copy_simple_kernel" if plan["simple_kernel"] else "kvm_copy_kernel")
-              + f"<u32x{plan['vector_bytes'] // 4}, {plan['threads']}, {plan['vectors_per_lane']}, "
-              + ("packed" if plan["pairs_per_launch"] > 432 else "wide") + ">")
-    traffic, traffic_source = measured_traffic(config if not (ctx_tp or fresh_pools) and pattern == "request" else 0,
-                                               kernel, bytes_per_launch)
     cache_resident = 2 * hbm_bytes <= INFINITY_CACHE_BYTES
-    out = {
-        "metric": "KV migration GB/s (% of HBM peak) + us/request at LLaMA-2-7B shape" if config == 2
-                  else f"KV migration GB/s (% of HBM peak) + us/request, {w.name}",
-        "value": round(hbm_gbps, 2), "unit": "GB/s",
-        "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": round(ms_per_step, 4),
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u8", "data": "synthetic",
-        "config": {
-            "workload": (f"{w.name}: {len(w.calls)} requests, {w.total_blocks} blocks of "
-                         f"{w.payload_bytes_per_block} B (K+V, decoding rank's share), context pp{w.ctx_pp}/tp{w.ctx_tp}"
-                         f" -> decoding pp{w.dec_pp}/tp{w.dec_tp} rank ({w.dec_pp_rank},{w.dec_tp_rank}), "
-                         f"pools {w.src_blocks}/{w.dst_blocks} blocks, seed {w.seed}"),
-            "pattern": ("one call per request" if pattern == "request" else
-                        f"{len(calls)} calls per batch (requests merged until a block id recurs)" if len(calls) > 1
-                        else "one call per batch"),
-            "value_counts": "HBM bytes read + written (2 x payload) per second",
-            "tuning": tuning,
-        },
-        "ms_per_step_median": round(per_step_ms[len(per_step_ms) // 2], 4), "ms_per_step_min": round(per_step_ms[0], 4),
-        "payload_GBps": round(payload / (ms_per_step * 1e-3) / 1e9, 2),
-        "frac_of_hbm_peak": round(hbm_gbps / HBM_PEAK_GBPS, 4),
-        "us_per_request": round(ms_per_step * 1e3 / len(w.calls), 2),
-        "blocks_per_s": round(w.total_blocks / (ms_per_step * 1e-3), 1),
-        "host_call_us": host_call_us, "host_call_us_min": host_call_us_min,
-        "bit_exact": bit_exact,
-        "roofline": {
-            "bound": "hbm", "achieved": round(bytes_per_launch / (launch_us * 1e-6) / 1e9, 2), "peak": HBM_PEAK_GBPS,
-            "unit": "GB/s", "frac": round(bytes_per_launch / (launch_us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
-            "traffic": traffic, "traffic_source": traffic_source,
-            "kernel": kernel,
-            "launches_per_step": launches_per_step,
-            "avg_launch_us": round(launch_us, 2), "algorithmic_bytes_per_launch": round(bytes_per_launch),
-            "workgroups_per_block": plan["workgroups_per_block"], "workgroup_size": plan["threads"],
-        },
-    }
-    if cache_resident:
-        # a step's reads and writes fit the 256 MB last-level cache and the steps repeat them:
-        # the figure is a cache and launch-latency figure, not an HBM one
-        out["cache_resident"] = True
-    if copy_ceiling is not None:
-        out["plain_copy_GBps"] = copy_ceiling
+    records = []
+    for pattern in patterns:
+        if records:
+            # the next pattern must write every block itself
+            dst_k.view(torch.int16).fill_(workloads.CANARY_BITS)
+            dst_v.view(torch.int16).fill_(workloads.CANARY_BITS)
+        calls = [(cabi.index_array(ci), cabi.index_array(di)) for ci, di in make_calls(w, pattern)]
+        plan = cabi.migrate_plan(geom, max(len(c[0]) for c in calls), dst_k.data_ptr(), dst_v.data_ptr(), w.dst_blocks)
+        launches_per_step = 0
+        for ci, _ in calls:
+            launches_per_step += cabi.migrate_plan(geom, len(ci), dst_k.data_ptr(), dst_v.data_ptr(),
+                                                   w.dst_blocks)["launches"]
+
+        def step():
+            for ci, di in calls:
+                cabi.migrate(geom, ci, di, dst_k.data_ptr(), dst_v.data_ptr(), w.dst_blocks, stream.cuda_stream)
+
+        for _ in range(warmup):
+            step()
+        # no collector pass inside the timed region (a full one over torch's modules takes 35 ms)
+        gc.collect()
+        gc.freeze()
+        torch.cuda.synchronize()
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record(stream)
+        for _ in range(steps):
+            step()
+        stop.record(stream)
+        torch.cuda.synchronize()
+        elapsed_ms = start.elapsed_time(stop)
+        ms_per_step = elapsed_ms / steps
+
+        # a second pass with an event between steps, for the spread (median and best step)
+        marks = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
+        marks[0].record(stream)
+        for i in range(steps):
+            step()
+            marks[i + 1].record(stream)
+        torch.cuda.synchronize()
+        per_step_ms = sorted(marks[i].elapsed_time(marks[i + 1]) for i in range(steps))
+
+        hbm_gbps = hbm_bytes / (ms_per_step * 1e-3) / 1e9
+        launch_us = elapsed_ms * 1e3 / (steps * launches_per_step)
+        bytes_per_launch = hbm_bytes / launches_per_step
+
+        bit_exact = verify(w, src_k, src_v, dst_k, dst_v) if verify_result else None
+        host_call_us, host_call_us_min = host_call_cost_us(cabi, geom, w, dst_k, dst_v, stream)
+
+        tuning = {"threads": plan["threads"], "vectors_per_lane": plan["vectors_per_lane"],
+                  "pairs_per_launch": plan["pairs_per_launch"],
+                  **{k: cabi.get_option(k) for k in ("xcd_map", "sort_pairs")}}
+        # the name the kernel trace shows, shortened: vector type, lanes, vectors per lane, index-table form
+        kernel = (("kvm_copy_simple_kernel" if plan["simple_kernel"] else "kvm_copy_kernel")
+                  + f"<u32x{plan['vector_bytes'] // 4}, {plan['threads']}, {plan['vectors_per_lane']}, "
+                  + ("packed" if plan["pairs_per_launch"] > 432 else "wide") + ">")
+        traffic, traffic_source = measured_traffic(
+            config if not (ctx_tp or fresh_pools) and pattern == "request" else 0, kernel, bytes_per_launch)
+        out = {
+            "metric": "KV migration GB/s (% of HBM peak) + us/request at LLaMA-2-7B shape" if config == 2
+                      else f"KV migration GB/s (% of HBM peak) + us/request, {w.name}",
+            "value": round(hbm_gbps, 2), "unit": "GB/s",
+            "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": round(ms_per_step, 4),
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u8", "data": "synthetic",
+            "config": {
+                "workload": (f"{w.name}: {len(w.calls)} requests, {w.total_blocks} blocks of "
+                             f"{w.payload_bytes_per_block} B (K+V, decoding rank's share), context pp{w.ctx_pp}/tp{w.ctx_tp}"
+                             f" -> decoding pp{w.dec_pp}/tp{w.dec_tp} rank ({w.dec_pp_rank},{w.dec_tp_rank}), "
+                             f"pools {w.src_blocks}/{w.dst_blocks} blocks, seed {w.seed}"),
+                "pattern": ("one call per request" if pattern == "request" else
+                            f"{len(calls)} calls per batch (requests merged until a block id recurs)" if len(calls) > 1
+                            else "one call per batch"),
+                "value_counts": "HBM bytes read + written (2 x payload) per second",
+                "tuning": tuning,
+            },
+            "ms_per_step_median": round(per_step_ms[len(per_step_ms) // 2], 4),
+            "ms_per_step_min": round(per_step_ms[0], 4),
+            "payload_GBps": round(payload / (ms_per_step * 1e-3) / 1e9, 2),
+            "frac_of_hbm_peak": round(hbm_gbps / HBM_PEAK_GBPS, 4),
+            "us_per_request": round(ms_per_step * 1e3 / len(w.calls), 2),
+            "blocks_per_s": round(w.total_blocks / (ms_per_step * 1e-3), 1),
+            "host_call_us": host_call_us, "host_call_us_min": host_call_us_min,
+            "bit_exact": bit_exact,
+            "roofline": {
+                "bound": "hbm", "achieved": round(bytes_per_launch / (launch_us * 1e-6) / 1e9, 2), "peak": HBM_PEAK_GBPS,
+                "unit": "GB/s", "frac": round(bytes_per_launch / (launch_us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
+                "traffic": traffic, "traffic_source": traffic_source,
+                "kernel": kernel,
+                "launches_per_step": launches_per_step,
+                "avg_launch_us": round(launch_us, 2), "algorithmic_bytes_per_launch": round(bytes_per_launch),
+                "workgroups_per_block": plan["workgroups_per_block"], "workgroup_size": plan["threads"],
+            },
+        }
+        if cache_resident:
+            # a step's reads and writes fit the 256 MB last-level cache and the steps repeat them:
+            # the figure is a cache and launch-latency figure, not an HBM one
+            out["cache_resident"] = True
+        records.append(out)
+    if calibrate_copy:
+        records[0]["plain_copy_GBps"] = time_plain_copy(cabi, stream)
     del src_k, src_v, dst_k, dst_v
     cabi.reset()
+    gc.unfreeze()
     torch.cuda.empty_cache()
-    return out, w
+    return records, w
 
 
 def compact(d: dict) -> dict:
@@ -399,45 +412,50 @@ def main():
         return
 
     if args.pattern.startswith(("handoff", "scheduler")):
+        if args.request_blocks:
+            print(json.dumps(run_handoff_by_size(args)))
+            return
         print(json.dumps(run_handoff_bench(args, load_workload(args.config or 2))))
         return
 
     verify_result = not args.no_verify
     if args.config:
         # one configuration, nothing else launched: the command the kernel profiles are taken with
-        out, w = bench_migrate(args.config, args.pattern, args.steps, args.warmup, verify_result,
-                               args.calibrate_copy, args.ctx_tp, args.fresh_pools)
+        (out,), w = bench_migrate(args.config, [args.pattern], args.steps, args.warmup, verify_result,
+                                  args.calibrate_copy, args.ctx_tp, args.fresh_pools)
         if not args.no_cpu_baseline:
             out["cpu_baseline"] = cpu_baseline(w)
         print(json.dumps(out))
         return
 
-    # The default run: configuration 2, one call per request, is the headline; every other
-    # configuration follows in its own pools and rides along in "configs".
-    out, w2 = bench_migrate(2, "request", args.steps, args.warmup, verify_result, args.calibrate_copy)
-    configs = {}
-    # every entry below rides along: one that fails says so in its place and costs neither the
-    # headline above nor the entries after it
+    # The default run: configuration 2, one call per request, is the headline; its batched form
+    # (same pools) and every other configuration (own pools, both call patterns on them) ride
+    # along in "configs".  An entry that fails says so in its place and costs neither the
+    # headline nor the entries after it.
     def failed(e):
         import torch as _torch
 
         _torch.cuda.empty_cache()
         return {"error": f"{type(e).__name__}: {e}"}
 
-    cpu_of = {}
-    for cfg, pattern in ((2, "batch"), (1, "request"), (3, "request"), (3, "batch"), (4, "request"), (4, "batch")):
-        key = f"cfg{cfg}" if pattern == "request" else f"cfg{cfg}_batched"
+    configs, cpu_of = {}, {}
+    (out, batched2), w2 = bench_migrate(2, ["request", "batch"], args.steps, args.warmup, verify_result, args.calibrate_copy)
+    configs["cfg2_batched"] = batched2
+    for cfg, patterns in ((1, ["request"]), (3, ["request", "batch"]), (4, ["request", "batch"])):
+        keys = [f"cfg{cfg}" if pattern == "request" else f"cfg{cfg}_batched" for pattern in patterns]
         try:
-            d, w = bench_migrate(cfg, pattern, args.steps, args.warmup, verify_result)
+            records, w = bench_migrate(cfg, patterns, args.steps, args.warmup, verify_result)
             if not args.no_cpu_baseline:
                 # every configuration's own CPU figure, on a sample that a few seconds cover; the
                 # two patterns of a configuration move the same bytes on the host and share it
-                if cfg not in cpu_of:
-                    cpu_of[cfg] = cpu_baseline(w, budget_s=2.5, max_blocks=64, max_payload_bytes=256 << 20)
-                d["cpu_baseline"] = cpu_of[cfg]
-            configs[key] = compact(d)
+                cpu_of[cfg] = cpu_baseline(w, budget_s=2.5, max_blocks=64, max_payload_bytes=256 << 20)
+            for key, d in zip(keys, records):
+                if cfg in cpu_of:
+                    d["cpu_baseline"] = cpu_of[cfg]
+                configs[key] = compact(d)
         except Exception as e:      # noqa: BLE001
-            configs[key] = failed(e)
+            for key in keys:
+                configs[key] = failed(e)
     try:
         configs["cfg5"] = run_swap_bench(args, default_only=True)
     except Exception as e:          # noqa: BLE001
@@ -470,8 +488,8 @@ def main():
     out["configs"] = configs
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(w2)
-        if "cfg2_batched" in configs and "error" not in configs["cfg2_batched"]:
-            configs["cfg2_batched"]["cpu_baseline"] = out["cpu_baseline"]
+        configs["cfg2_batched"]["cpu_baseline"] = out["cpu_baseline"]
+    configs["cfg2_batched"] = compact(configs["cfg2_batched"])
     print(json.dumps(out))
 
 
@@ -1100,12 +1118,20 @@ def run_handoff_bench(args, w):
     ms_per_step = total_s / args.steps * 1e3
     hbm_gbps = 2 * w.payload_bytes / (ms_per_step * 1e-3) / 1e9
     cabi.reset()
+    # the engines were frozen into the collector's permanent generation with everything else;
+    # thaw and collect, or their pools (cycles hold them) stay allocated for the rest of the run
+    driven_by_scheduler = sched is not None
+    del src_k, src_v, dw, sched
+    ctx.workers, dec.workers = [], []
+    gc.unfreeze()
+    gc.collect()
+    torch.cuda.empty_cache()
     return {
         "metric": f"KV migration hand-off GB/s + us/request, {w.name}", "value": round(hbm_gbps, 2), "unit": "GB/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u8", "data": "synthetic",
         "config": {"workload": f"{w.name}: {len(w.calls)} requests, {w.total_blocks} blocks",
-                   "pattern": (("bridge queue -> DecodingStageFCFSScheduler.post_process -> " if sched is not None else "")
+                   "pattern": (("bridge queue -> DecodingStageFCFSScheduler.post_process -> " if driven_by_scheduler else "")
                                + "BlockManager.allocate_blocks + Worker.migrate_blocks (torch op) + release of the "
                                "context blocks, " + ("one migrate call per batch" if batched else "one per request")),
                    "value_counts": "HBM bytes read + written per second of host wall clock (allocation to GPU idle)"},
@@ -1119,6 +1145,60 @@ def run_handoff_bench(args, w):
         "frac_of_hbm_peak": round(hbm_gbps / HBM_PEAK_GBPS, 4),
         "block_tables_equal_workload": same_tables, "bit_exact": bit_exact,
     }
+
+
+def run_handoff_by_size(args):
+    """The hand-off pattern over requests of one size, for every size asked for: per request
+    the wall clock to GPU idle, the host's share, where the host's share goes, and beside
+    them the copy alone (the same block lists through the C ABI, HIP events) -- so that it
+    shows from which prompt length on the GPU, not the host, is the longer leg."""
+    import torch
+
+    from distserve_amd import cabi, workloads
+
+    by_size = {}
+    for n in args.request_blocks:
+        w = workloads.fixed_size_requests(n)
+        h = run_handoff_bench(args, w)
+        # the copy alone: same lists, one call per request, nothing but the launches timed
+        s = w.shape
+        src_k = workloads.fill_uniform(w.src_pool_shape(), 1, "cuda")
+        src_v = workloads.fill_uniform(w.src_pool_shape(), 2, "cuda")
+        dst_k, dst_v = torch.empty_like(src_k), torch.empty_like(src_v)
+        cabi.reset()
+        cabi.register_source(1, 1, 0, 0, s.num_layers, s.num_kv_heads, src_k.data_ptr(), src_v.data_ptr(),
+                             src_k.numel() * s.dtype_bytes)
+        geom = cabi.geom(s.num_layers, s.num_kv_heads, s.block_size, s.head_dim, s.dtype_bytes)
+        calls = [(cabi.index_array(c.ctx_idx), cabi.index_array(c.dec_idx)) for c in w.calls]
+        stream = torch.cuda.current_stream()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        for timed in (False, True):
+            e0.record(stream)
+            for _ in range(args.steps):
+                for ci, di in calls:
+                    cabi.migrate(geom, ci, di, dst_k.data_ptr(), dst_v.data_ptr(), w.dst_blocks, stream.cuda_stream)
+            e1.record(stream)
+            torch.cuda.synchronize()
+        copy_us = e0.elapsed_time(e1) * 1e3 / (args.steps * len(calls))
+        cabi.reset()
+        del src_k, src_v, dst_k, dst_v
+        torch.cuda.empty_cache()
+        by_size[str(n)] = {
+            "prompt_tokens": n * s.block_size, "requests_per_step": len(w.calls),
+            "us_per_request": h["us_per_request"], "host_us_per_request": h["host_us_per_request"],
+            "host_us_per_request_by_step": h["host_us_per_request_by_step"],
+            "copy_alone_us_per_request": round(copy_us, 2), "GBps": h["value"], "bit_exact": h["bit_exact"],
+            "block_tables_equal_workload": h["block_tables_equal_workload"],
+            "longer_leg": "host" if h["host_us_per_request"] > copy_us else "gpu"}
+    first = by_size[str(args.request_blocks[0])]
+    return {"metric": "KV migration hand-off us/request by request size, LLaMA-2-7B shape", "value": first["us_per_request"],
+            "unit": "us/request", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+            "ms_per_step": round(first["us_per_request"] * first["requests_per_step"] * 1e-3, 4),
+            "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "u8", "data": "synthetic",
+            "config": {"workload": "48 requests of N blocks each (8 MiB per block, K+V), scattered block lists, TP1 -> TP1; "
+                                   f"value is N = {args.request_blocks[0]}",
+                       "pattern": args.pattern},
+            "by_request_blocks": by_size}
 
 
 def verify(w, src_k, src_v, dst_k, dst_v) -> bool:

