@@ -469,6 +469,86 @@ def test_calls_from_several_host_threads_on_their_own_streams(kvm):
     kvm.reset()
 
 
+def test_registrations_from_one_thread_while_others_migrate(kvm):
+    """A decoding worker may bind a second context instance (and re-bind it, and bind ranks it
+    never reads) while its migrations from the first one are running on other threads: the
+    registry is read under a shared lock and changed under an exclusive one, and a migration
+    always sees the pools of a whole registration."""
+    import threading
+
+    g = oracle.Geom(2, 4, 16, 64, 2)
+    kvm.reset()
+    nb = 48
+    src_k, src_v = make_src_pools(g, nb, 51), make_src_pools(g, nb, 52)
+    keep = upload_and_register(g, src_k, src_v)                     # context instance 0
+    other_k, other_v = make_src_pools(g, nb, 61), make_src_pools(g, nb, 62)
+    dev_other = (other_k[0][0].cuda(), other_v[0][0].cuda())
+    stop, errors, results = threading.Event(), [], {}
+
+    def register():
+        try:
+            torch.cuda.set_device(0)
+            n = 0
+            while not stop.is_set():
+                for inst in (1, 2, 3):
+                    kvm.register_source(1, 1, 0, 0, g.num_layers, g.num_kv_heads, dev_other[0].data_ptr(),
+                                        dev_other[1].data_ptr(), dev_other[0].numel() * 2, ctx_instance=inst)
+                h = kvm.get_mem_handle(dev_other[0].data_ptr(), dev_other[0].numel() * 2)
+                kvm.register_mem_handle(h, h, g.num_layers, g.num_kv_heads, [1, 0, 1, 0], [1, 0, 1, 0], ctx_instance=4)
+                n += 1
+            results["registrations"] = n
+        except Exception as e:      # noqa: BLE001
+            errors.append(("register", repr(e)))
+
+    def work(tid):
+        try:
+            torch.cuda.set_device(0)
+            stream = torch.cuda.Stream()
+            gen = torch.Generator().manual_seed(200 + tid)
+            dk = canary_pool(g.dec_pool_shape(nb)).cuda()
+            dv = canary_pool(g.dec_pool_shape(nb)).cuda()
+            calls = []
+            for _ in range(200):
+                n = int(torch.randint(1, 9, (1,), generator=gen))
+                ci = torch.randint(0, nb, (n,), generator=gen).tolist()
+                di = torch.randperm(nb, generator=gen)[:n].tolist()
+                kvm.migrate(kvm_geom(g), ci, di, dk.data_ptr(), dv.data_ptr(), nb, stream.cuda_stream)
+                calls.append((ci, di))
+            stream.synchronize()
+            results[tid] = (dk.cpu(), dv.cpu(), calls)
+        except Exception as e:      # noqa: BLE001
+            errors.append((tid, repr(e)))
+
+    registrar = threading.Thread(target=register)
+    workers = [threading.Thread(target=work, args=(t,)) for t in range(3)]
+    registrar.start()
+    for t in workers:
+        t.start()
+    for t in workers:
+        t.join()
+    stop.set()
+    registrar.join()
+    assert not errors, errors
+    assert results["registrations"] >= 1
+    for tid in range(3):
+        dk, dv, calls = results[tid]
+        want_k, want_v = canary_pool(g.dec_pool_shape(nb)), canary_pool(g.dec_pool_shape(nb))
+        for ci, di in calls:
+            oracle.migrate_c(g, src_k, ci, di, want_k)
+            oracle.migrate_c(g, src_v, ci, di, want_v)
+        assert same_bits(dk, want_k) and same_bits(dv, want_v), tid
+    # the instance bound meanwhile is usable afterwards
+    g1 = kvm.geom(g.num_layers, g.num_kv_heads, g.block_size, g.head_dim, g.dtype_bytes, ctx_instance=1)
+    dk, dv = canary_pool(g.dec_pool_shape(nb)).cuda(), canary_pool(g.dec_pool_shape(nb)).cuda()
+    kvm.migrate(g1, [5, 7], [0, 1], dk.data_ptr(), dv.data_ptr(), nb, stream_handle())
+    torch.cuda.synchronize()
+    want_k, want_v = oracle_migrate(g, other_k, other_v, [5, 7], [0, 1], nb)
+    assert same_bits(dk.cpu(), want_k) and same_bits(dv.cpu(), want_v)
+    assert kvm.opened_handles() == 0
+    del keep
+    kvm.reset()
+
+
 @pytest.mark.parametrize("make", [
     workloads.config3, workloads.config4,
     functools.partial(workloads.config3, fresh_pools=True), functools.partial(workloads.config4, fresh_pools=True),
