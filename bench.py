@@ -504,6 +504,7 @@ def run_swap_bench(args, default_only: bool = False):
     import torch
 
     from distserve_amd import cabi, workloads
+    from distserve_amd.streams import side_streams
 
     torch.cuda.set_device(0)
     kw = {}
@@ -515,7 +516,7 @@ def run_swap_bench(args, default_only: bool = False):
     w = workloads.config5(**kw)
     shape = w.shape
     main = torch.cuda.current_stream()
-    out_stream, in_stream = torch.cuda.Stream(), torch.cuda.Stream()
+    out_stream, in_stream = side_streams(2)            # two that do not share a hardware queue
 
     k_gpu = workloads.fill_uniform(shape.pool_shape(w.gpu_blocks), w.seed, "cuda")
     v_gpu = workloads.fill_uniform(shape.pool_shape(w.gpu_blocks), w.seed + 500, "cuda")

@@ -55,7 +55,10 @@ class _Shelf:
             call_workers(self.flush_call)
             self.free += self.quarantine
             self.quarantine = []
-        taken, self.free = self.free[:count], self.free[count:]
+        # the head of the list, cut off in place: slicing the rest into a new list would copy (and
+        # re-count) every free block of the pool on every allocation, microseconds per call
+        taken = self.free[:count]
+        del self.free[:count]
         return taken
 
     def used(self) -> int:

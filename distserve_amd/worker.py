@@ -25,7 +25,12 @@ import torch
 
 from distserve_amd.config import CacheConfig, ModelConfig, ParallelConfig
 from distserve_amd.request import Request
+from distserve_amd.streams import side_streams
 from distserve_amd.utils import MemoryHandle, Stage
+
+
+# torch's accessor of the current stream's raw handle (an int), where this build of torch has it
+_RAW_STREAM = getattr(torch._C, "_cuda_getCurrentRawStream", None)
 
 
 def _require_gpu() -> None:
@@ -47,6 +52,7 @@ class MigrationMark:
 
     def __init__(self, stream: torch.cuda.Stream, eager: bool = False):
         self.stream = stream
+        self.raw_stream = stream.cuda_stream   # the hipStream_t as an int: what the hot path compares
         self._event: Optional[torch.cuda.Event] = None
         if eager:
             self._recorded()
@@ -92,7 +98,9 @@ class Worker:
         self.forward = forward
         self.device = torch.device("cuda:0")
         torch.cuda.set_device(self.device)
+        self._device_index = self.device.index
         self._default_stream = torch.cuda.default_stream(self.device)
+        self._default_raw_stream = self._default_stream.cuda_stream
         # the overloads, resolved once: a lookup through torch.ops per call costs microseconds
         self._migrate_op = torch.ops.block_migration_ops.migrate_blocks_from.default
         self._swap_op = torch.ops.swapping_ops.swap.default
@@ -101,9 +109,10 @@ class Worker:
         self.v_cache: Optional[torch.Tensor] = None
         self.k_swap: Optional[torch.Tensor] = None    # same block shape, pinned host memory
         self.v_swap: Optional[torch.Tensor] = None
-        # default-priority side streams, one per direction (reference worker.py:64-66)
-        self.swap_in_stream = torch.cuda.Stream()
-        self.swap_out_stream = torch.cuda.Stream()
+        # default-priority side streams, one per direction (reference worker.py:64-66), picked so
+        # that the GPU runs them beside each other and beside the default stream: two streams
+        # that share a hardware queue would turn a swap-out and a swap-in into one after the other
+        self.swap_in_stream, self.swap_out_stream = side_streams(2, device=self.device)
         self.swap_event_table: Dict[int, torch.cuda.Event] = {}   # request_id -> its latest swap
         self.latest_swap_in_event: Optional[torch.cuda.Event] = None
         self.latest_swap_out_event: Optional[torch.cuda.Event] = None
@@ -118,6 +127,13 @@ class Worker:
         # with the device named, torch does not re-count the devices on every call (tens of
         # microseconds each on ROCm), which matters for a call made once per migrated request
         return torch.cuda.current_stream(self.device)
+
+    def _current_raw_stream(self) -> int:
+        """The current stream's hipStream_t as an int, without building a Stream object
+        (1-2 microseconds each, twice per migrated request otherwise)."""
+        if _RAW_STREAM is not None:
+            return _RAW_STREAM(self._device_index)
+        return self._current_stream().cuda_stream
 
     # ---- pools
 
@@ -217,17 +233,20 @@ class Worker:
             self.k_cache,
             self.v_cache,
         )
-        stream = self._current_stream()
+        raw = self._current_raw_stream()
         mark = self.latest_migrate_event
         # a mark on the same stream that nobody has asked for an event yet stands for these copies too
-        if mark is None or not mark.pending or mark.stream != stream:
-            self.latest_migrate_event = MigrationMark(stream, eager=stream != self._default_stream)
+        if mark is None or mark.raw_stream != raw or not mark.pending:
+            self.latest_migrate_event = MigrationMark(self._current_stream(), eager=raw != self._default_raw_stream)
 
     def wait_stream_for_migration(self, event: Optional[MigrationMark]) -> None:
         """Called on a *context* worker: work it enqueues from now on (the next prefill that
         may overwrite freed blocks) runs after the migration that read them."""
-        if event is not None:
-            event.wait(self._current_stream())
+        if event is None:
+            return
+        if getattr(event, "raw_stream", None) == self._current_raw_stream():
+            return                      # the same stream: behind the copies by stream order alone
+        event.wait(self._current_stream())
 
     # ---- swap
 
