@@ -485,6 +485,15 @@ def main():
         configs["cfg2_handoff"].update(GBps=h["value"], pattern=h["config"]["pattern"])
     except Exception as e:      # noqa: BLE001
         configs["cfg2_handoff"] = failed(e)
+    # ... and by request size: below which prompt length the host, not the GPU, is the longer leg
+    try:
+        hand.pattern, hand.request_blocks = "handoff", [1, 4, 16]
+        rows = run_handoff_by_size(hand)["by_request_blocks"]
+        configs["cfg2_handoff"]["by_request_blocks"] = {
+            n: {k: r[k] for k in ("prompt_tokens", "us_per_request", "host_us_per_request", "copy_alone_us_per_request",
+                                  "longer_leg", "bit_exact")} for n, r in rows.items()}
+    except Exception as e:      # noqa: BLE001
+        configs["cfg2_handoff"]["by_request_blocks"] = failed(e)
     out["configs"] = configs
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(w2)

@@ -79,6 +79,13 @@ def test_migration_line_meets_the_contract_and_the_target():
     hand = configs["cfg2_handoff"]
     assert hand["bit_exact"] is True and hand["block_tables_equal_workload"] is True and hand["frac_of_hbm_peak"] >= 0.70
     assert hand["transmission_us_per_request"] > hand["transmission_us_per_request_stamped_at_enqueue"] > 0
+    by_size = hand["by_request_blocks"]
+    assert sorted(by_size) == ["1", "16", "4"], by_size
+    for n, r in by_size.items():
+        assert r["bit_exact"] is True and r["prompt_tokens"] == 16 * int(n), (n, r)
+        assert 0 < r["host_us_per_request"] <= r["us_per_request"], (n, r)
+    assert by_size["16"]["longer_leg"] == "gpu" and by_size["16"]["host_us_per_request"] < 30, \
+        f"performance, not correctness: {by_size['16']}"
     assert configs["cfg2_ipc"].get("bit_exact") is True, configs["cfg2_ipc"]
     assert configs["cfg2_ipc"]["other_over_this_process"] >= 0.85, \
         f"performance, not correctness: pools of another process at {configs['cfg2_ipc']}"
