@@ -58,6 +58,8 @@ def parse_args():
     ap.add_argument("--ipc-child", action="store_true", help=argparse.SUPPRESS)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-verify", action="store_true")
+    ap.add_argument("--kernel-digest", action="store_true",
+                    help="print the digest of the kernels' source (what a counter summary under profiles/ records) and exit")
     ap.add_argument("--opt", action="append", default=[], help="kvmove tuning option name=value")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also time the plain contiguous copy kernel (adds launches to a profile)")
@@ -75,14 +77,29 @@ def parse_args():
     return ap.parse_args()
 
 
+def kernel_source_digest() -> str:
+    """First 16 hex digits of the SHA-256 of the kernels' source: the text of kvmove.hip from
+    the kernel-argument layout to the end of the device code (host-side edits do not change
+    it).  A counter summary under profiles/ carries the digest of the source it was taken
+    with (``KERNEL_SOURCE_DIGEST``; ``python3 bench.py --kernel-digest`` prints it)."""
+    import hashlib
+
+    text = open(os.path.join(ROOT, "distserve_amd", "csrc", "kvmove.hip")).read()
+    begin = text.index("// ------------------------------------------------------------------ kernel argument")
+    end = text.index("// --------------------------------------------------------------------------- host")
+    return hashlib.sha256(text[begin:end].encode()).hexdigest()[:16]
+
+
 def measured_traffic(config: int, kernel: str, algorithmic_bytes_per_launch: float):
     """(HBM bytes per launch, where the figure comes from).  Hardware counters cannot be read
     inside this run: the ratio of counted to algorithmic bytes is taken from the committed
     counter summary of this configuration's kernel (two rocprofv3 --pmc runs, FETCH_SIZE and
     WRITE_SIZE, each scaled by a plain copy of known size) and applied to this run's
     algorithmic bytes.  The summary names the kernel it was taken with (a line
-    ``KERNEL_OF_RECORD <name>``); (None, why) when no summary has been committed for the
-    configuration or when it is of another kernel than this run's."""
+    ``KERNEL_OF_RECORD <name>``) and the digest of the kernel source it was built from
+    (``KERNEL_SOURCE_DIGEST``); (None, why) when no summary has been committed for the
+    configuration, when it is of another kernel than this run's, or when the kernels' source
+    has changed since."""
     import re
 
     name = f"profiles/kvm_copy_kernel_cfg{config}_pmc.txt"
@@ -94,6 +111,10 @@ def measured_traffic(config: int, kernel: str, algorithmic_bytes_per_launch: flo
     if not of_record or of_record.group(1).strip() != kernel:
         return None, (f"{name} was taken with {of_record.group(1).strip() if of_record else 'an unnamed kernel'}, "
                       f"this run used {kernel}: not applied")
+    digest = re.search(r"^KERNEL_SOURCE_DIGEST ([0-9a-f]+)$", text, flags=re.M)
+    if not digest or digest.group(1) != kernel_source_digest():
+        return None, (f"{name} was taken with kernel source {digest.group(1) if digest else '(no digest)'}, "
+                      f"this tree's is {kernel_source_digest()}: not applied")
     m = re.search(r"TRAFFIC_PER_ALGORITHMIC_BYTE read=([0-9.]+) write=([0-9.]+)", text)
     if not m:
         return None, None
@@ -374,6 +395,9 @@ def compact(d: dict) -> dict:
 
 def main():
     args = parse_args()
+    if args.kernel_digest:
+        print(kernel_source_digest())
+        return
     if args.ipc_child:
         run_ipc_child()
         return

@@ -48,3 +48,28 @@ def test_only_tests_smoke_and_the_cpu_baseline_import_the_oracle():
         head = bench[:match.start()]
         owner = re.findall(r"^def (\w+)", head, re.M)[-1]
         assert "cpu_baseline" in owner, owner
+
+
+def test_counter_summaries_are_of_the_kernels_as_they_are_now():
+    """The traffic ratio bench.py reports comes from committed counter summaries; each names the
+    kernel it was taken with and the digest of the kernel source it was built from.  A change
+    to the kernels without new counter runs fails here (and makes bench.py report no traffic)."""
+    import importlib.util
+    import re
+
+    spec = importlib.util.spec_from_file_location("bench_for_digest", os.path.join(ROOT, "bench.py"))
+    bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bench)
+    now = bench.kernel_source_digest()
+    assert re.fullmatch(r"[0-9a-f]{16}", now)
+    for config in (2, 3, 4):
+        path = os.path.join(ROOT, "profiles", f"kvm_copy_kernel_cfg{config}_pmc.txt")
+        text = open(path).read()
+        of_record = re.search(r"^KERNEL_OF_RECORD (.+)$", text, flags=re.M)
+        digest = re.search(r"^KERNEL_SOURCE_DIGEST ([0-9a-f]+)$", text, flags=re.M)
+        assert of_record and digest, path
+        assert digest.group(1) == now, f"{path} was taken with other kernel source: take the counters again"
+        traffic, source = bench.measured_traffic(config, of_record.group(1).strip(), 1e9)
+        assert traffic is not None and 0.99e9 < traffic < 1.05e9 and "profiles/" in source
+        # another kernel's name is refused
+        assert bench.measured_traffic(config, "some_other_kernel", 1e9)[0] is None
